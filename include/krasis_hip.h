@@ -352,6 +352,77 @@ size_t kr_decode_device_bytes(const kr_decode_store* s);
  *        8 route_select 9 moe_w13 10 moe_w2 11 moe_combine 12 lm_head 13 argmax 14 shared-gate matvec */
 int kr_decode_profile_step(kr_decode_store* s, int token_id, int position, double* ms_by_kind, long* launches_by_kind, int n_kinds);
 
+/* ================================================================================================
+ * Batched serving store: several requests decode / take prompt portions in ONE step.  No counterpart in the reference's single-request engines;
+ * it serves model designs whose weights stay in bf16 (or f32) and whose layers are described by kr_serve_layer.  Weights, GEMM inputs and cache rows
+ * are stored in `dtype`; positions, rotation angles, norms, the router, attention scores / weights and the residual stream are f32 in both.
+ * The cache is a pool of pages of `page_tokens` positions shared by `max_slots` request slots; a slot's pages are taken from the pool as its
+ * request grows and go back to it on release.  A step takes, per entry, a slot and the request's next tokens (any count >= 1), runs them from the
+ * cache earlier steps left, and returns the logits of the rows asked for.
+ * ================================================================================================ */
+typedef struct kr_serve kr_serve;
+#define KR_SERVE_BF16 0
+#define KR_SERVE_F32 1
+#define KR_SERVE_NORM_LAYER 0   /* (x - mean) / sqrt(var + eps) * w + b */
+#define KR_SERVE_NORM_RMS 1     /* x / sqrt(mean(x^2) + eps) * w */
+#define KR_SERVE_MLP_NONE 0
+#define KR_SERVE_MLP_DENSE 1
+#define KR_SERVE_MLP_MOE 2
+#define KR_SERVE_ACT_GELU_TANH 0       /* gelu_tanh(gate) * up */
+#define KR_SERVE_ACT_CLAMPED_SWIGLU 1  /* g = min(gate, limit), u = clamp(up, +-limit): g * sigmoid(alpha g) * (u + 1) */
+#define KR_SERVE_ACT_SILU 2            /* silu(gate) * up */
+typedef struct {
+    int vocab, width, n_layers;
+    int dtype;                  /* KR_SERVE_BF16 | KR_SERVE_F32 */
+    int norm_kind; float norm_eps;
+    int max_slots, page_tokens, pool_tokens;   /* pool_tokens / page_tokens pages for all slots together */
+} kr_serve_config;
+typedef struct {
+    /* mixer: attention with a parallel feed-forward on the same normed input (x += mixer(h) + ff(h)) */
+    int heads, kv_heads, dim, vdim;
+    int rot_dims, rot_interleaved;     /* rotary on the first rot_dims of a head; pairs (2i, 2i + 1) or (i, i + rot_dims / 2) */
+    double rot_base, rot_factor;       /* f_i = base^(-2i / rot_dims) / factor */
+    int qk_unit_norm;                  /* q, k divided by their root mean square over dim after the rotation (eps = norm_eps) */
+    float scale;
+    int window;                        /* position i sees j with 0 <= i - j < window; 0 = all earlier positions */
+    int has_sink;                      /* softmax denominator + exp(sink[head]) */
+    int kv_from;                       /* -1, or the earlier layer whose cached keys / values this layer attends to (no k / v projections of its own) */
+    int mlp_kind;
+    int ff, dense_act;                 /* dense: down(act(gate h, up h)) */
+    int experts, top, groups, keep, renorm;   /* router: softmax over all experts; best `keep` of `groups` groups; `top` experts; weights = scores */
+    int expert_ff, expert_act; float expert_limit, expert_alpha;
+    int shared_ff; float shared_limit;        /* 0 = no shared expert */
+} kr_serve_layer;
+/* tensor roles of kr_serve_set_tensor; layer = -1 for the first four */
+enum { KR_SV_EMBED = 0, KR_SV_FINAL_NORM_W, KR_SV_FINAL_NORM_B, KR_SV_HEAD, KR_SV_NORM_W, KR_SV_NORM_B, KR_SV_Q, KR_SV_K, KR_SV_V, KR_SV_O, KR_SV_SINK,
+       KR_SV_GATE, KR_SV_UP, KR_SV_DOWN, KR_SV_ROUTER, KR_SV_EXPERT_GATE, KR_SV_EXPERT_UP, KR_SV_EXPERT_DOWN, KR_SV_SHARED_GATE, KR_SV_SHARED_UP,
+       KR_SV_SHARED_DOWN, KR_SV_N_ROLES };
+int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_serve_layer* layers, kr_serve** out);
+void kr_serve_destroy(kr_serve* s);
+/* host tensor [rows, cols] row-major ([out, in] for projections), src_dtype KR_SERVE_BF16 / KR_SERVE_F32; `index` = expert for the expert roles */
+int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void* host, int src_dtype, int rows, int cols);
+/* every tensor generated on the device: projections uniform in +-amp / sqrt(in), norm weights 1, biases and sinks 0 (benchmarks at sizes no checkpoint has) */
+int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp);
+int kr_serve_finalize(kr_serve* s);    /* refuses a store with a missing tensor */
+int kr_serve_admit(kr_serve* s, int* slot_out);          /* KR_ERR_STATE when every slot is live */
+int kr_serve_release(kr_serve* s, int slot);             /* the slot's pages return to the pool */
+int kr_serve_slot_len(kr_serve* s, int slot, int* len_out);
+int kr_serve_free_pages(kr_serve* s, int* n_out);
+/* One step.  tokens = the entries' tokens one after the other; want_rows index that array.  logits_out: host f32 [n_want, vocab] or NULL;
+ * argmax_out: host i32 [n_want] or NULL.  KR_ERR_STATE when the pool has too few free pages (nothing is changed then). */
+int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* counts, const int* tokens, int n_want, const int* want_rows, float* logits_out,
+                  int* argmax_out);
+/* the framework's sampler (kr_decode_sample's arithmetic) on wanted row `row` of the last step */
+int kr_serve_sample(kr_serve* s, int row, float temperature, int top_k, float top_p, uint64_t rng_seed, int* token_out);
+/* test aid: keep the residual stream after every layer of the next steps ([n_layers, T, width] f32), read it back */
+int kr_serve_set_capture(kr_serve* s, int enable);
+int kr_serve_read_capture(kr_serve* s, float* out_host, size_t n_floats);
+size_t kr_serve_device_bytes(const kr_serve* s);
+/* measurement hook: HIP-event time of every kernel family over the steps since the last reset (ms), families: 0 norm 1 gemm 2 qk_prep 3 attention 4 router+sort
+ * 5 activation 6 residual 7 embed / head rows / argmax */
+int kr_serve_set_profiling(kr_serve* s, int enable);
+int kr_serve_get_profile(kr_serve* s, double* ms_by_family, int n);
+
 /* ---- measurement hooks (bench.py): HIP events around each kernel launch on the launch stream ----
  * kinds: 0 kr_moe_w13_kernel, 1 kr_moe_w2_kernel, 2 kr_moe_combine_kernel.  Enabling profiling serialises calls. */
 int kr_set_profiling(kr_engine* e, int enable);

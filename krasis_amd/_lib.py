@@ -27,6 +27,9 @@ SYMBOLS = [
     "kr_decode_fused_add_rmsnorm", "kr_decode_rmsnorm", "kr_decode_silu_mul", "kr_decode_fused_shared_expert", "kr_decode_linear_attention_recurrent",
     "kr_decode_gated_rmsnorm_silu", "kr_decode_linear_attention_conv", "kr_decode_store_route_weight", "kr_decode_moe_route", "kr_decode_num_route_weights",
     "kr_decode_weight_bytes",
+    "kr_serve_create", "kr_serve_destroy", "kr_serve_set_tensor", "kr_serve_fill_synthetic", "kr_serve_finalize", "kr_serve_admit", "kr_serve_release",
+    "kr_serve_slot_len", "kr_serve_free_pages", "kr_serve_step", "kr_serve_sample", "kr_serve_set_capture", "kr_serve_read_capture", "kr_serve_device_bytes",
+    "kr_serve_set_profiling", "kr_serve_get_profile",
 ]
 TOKEN_CB = C.CFUNCTYPE(C.c_int, C.c_int, C.c_int, C.c_void_p)      # kr_token_cb(token, finish_reason, user) -> continue?
 
@@ -42,11 +45,85 @@ class ModelConfigC(C.Structure):
                 ("activation_alpha", C.c_float)]
 
 
+class ServeConfigC(C.Structure):
+    _fields_ = [("vocab", C.c_int), ("width", C.c_int), ("n_layers", C.c_int), ("dtype", C.c_int), ("norm_kind", C.c_int), ("norm_eps", C.c_float),
+                ("max_slots", C.c_int), ("page_tokens", C.c_int), ("pool_tokens", C.c_int)]
+
+
+class ServeLayerC(C.Structure):
+    _fields_ = [("heads", C.c_int), ("kv_heads", C.c_int), ("dim", C.c_int), ("vdim", C.c_int), ("rot_dims", C.c_int), ("rot_interleaved", C.c_int),
+                ("rot_base", C.c_double), ("rot_factor", C.c_double), ("qk_unit_norm", C.c_int), ("scale", C.c_float), ("window", C.c_int),
+                ("has_sink", C.c_int), ("kv_from", C.c_int), ("mlp_kind", C.c_int), ("ff", C.c_int), ("dense_act", C.c_int), ("experts", C.c_int),
+                ("top", C.c_int), ("groups", C.c_int), ("keep", C.c_int), ("renorm", C.c_int), ("expert_ff", C.c_int), ("expert_act", C.c_int),
+                ("expert_limit", C.c_float), ("expert_alpha", C.c_float), ("shared_ff", C.c_int), ("shared_limit", C.c_float)]
+
+
 _lib = None
+_serve_lib = None
+_SERVE_LIB = os.path.join(_HERE, "libkrasis_serve.so")
 
 
 def lib_path() -> str:
     return _LIB
+
+
+def _bind_serve(lib: C.CDLL) -> None:
+    vp, ci, cf = C.c_void_p, C.c_int, C.c_float
+    lib.kr_last_error.restype = C.c_char_p
+    lib.kr_serve_create.argtypes = [ci, C.POINTER(ServeConfigC), C.POINTER(ServeLayerC), C.POINTER(vp)]
+    lib.kr_serve_destroy.argtypes = [vp]; lib.kr_serve_destroy.restype = None
+    lib.kr_serve_set_tensor.argtypes = [vp, ci, ci, ci, vp, ci, ci, ci]
+    lib.kr_serve_fill_synthetic.argtypes = [vp, C.c_uint64, cf]
+    lib.kr_serve_finalize.argtypes = [vp]
+    lib.kr_serve_admit.argtypes = [vp, C.POINTER(ci)]
+    lib.kr_serve_release.argtypes = [vp, ci]
+    lib.kr_serve_slot_len.argtypes = [vp, ci, C.POINTER(ci)]
+    lib.kr_serve_free_pages.argtypes = [vp, C.POINTER(ci)]
+    lib.kr_serve_step.argtypes = [vp, ci, vp, vp, vp, ci, vp, vp, vp]
+    lib.kr_serve_sample.argtypes = [vp, ci, cf, ci, cf, C.c_uint64, C.POINTER(ci)]
+    lib.kr_serve_set_capture.argtypes = [vp, ci]
+    lib.kr_serve_read_capture.argtypes = [vp, vp, C.c_size_t]
+    lib.kr_serve_device_bytes.argtypes = [vp]; lib.kr_serve_device_bytes.restype = C.c_size_t
+    lib.kr_serve_set_profiling.argtypes = [vp, ci]
+    lib.kr_serve_get_profile.argtypes = [vp, C.POINTER(C.c_double), ci]
+
+
+def load_serve_library(build: bool = False) -> C.CDLL:
+    """The library that holds the batched serving store (kr_serve_*): libkrasis_hip.so when it is built, else libkrasis_serve.so -- the same
+    objects linked alone, which a checkout that only serves such models compiles in seconds (`make -C krasis_amd/csrc serve`; build=True runs it
+    when neither library is there).  torch, when the process already uses it, is imported first so that both bind one HIP runtime."""
+    global _serve_lib
+    if _serve_lib is not None:
+        return _serve_lib
+    if os.path.exists(_LIB):
+        full = load_library()
+        if hasattr(full, "kr_serve_create"):
+            _serve_lib = full
+            return full
+    if not os.path.exists(_SERVE_LIB):
+        if not build:
+            raise KrasisHipError(f"{_LIB} / {_SERVE_LIB} are missing: build with `make -C krasis_amd/csrc` (or `... serve`). krasis_amd has no CPU fallback.")
+        import subprocess
+        import sys
+        subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "serve"], stdout=sys.stderr)
+    import sys
+    if "torch" in sys.modules:
+        import torch  # noqa: F401
+    lib = C.CDLL(_SERVE_LIB)
+    _bind_serve(lib)
+    _serve_lib = lib
+    return lib
+
+
+def check_serve(rc: int) -> None:
+    if rc == KR_OK:
+        return
+    msg = load_serve_library().kr_last_error().decode("utf-8", "replace")
+    if rc == KR_ERR_STATE:
+        raise RuntimeError(msg)
+    if rc == KR_ERR_VALUE:
+        raise ValueError(msg)
+    raise KrasisHipError(msg)
 
 
 def load_library() -> C.CDLL:
@@ -164,6 +241,8 @@ def load_library() -> C.CDLL:
     lib.kr_decode_moe_route.argtypes = [vp, ci, vp, vp, vp, ci, ci, ci]
     lib.kr_decode_num_route_weights.argtypes = [vp]
     lib.kr_decode_weight_bytes.argtypes = [vp, ci]; lib.kr_decode_weight_bytes.restype = C.c_size_t
+    if hasattr(lib, "kr_serve_create"):
+        _bind_serve(lib)
     _lib = lib
     return lib
 

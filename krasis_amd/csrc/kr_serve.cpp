@@ -1,0 +1,521 @@
+// kr_serve.cpp -- the batched serving store behind kr_serve_* (include/krasis_hip.h): weights in bf16 or f32, a page pool shared by the request
+// slots, and the step function that runs a ragged batch (prompt portions beside single decoded tokens) through every layer.
+//
+// Memory: one K and one V pool per layer that owns a cache, [pages][page_tokens][kv_heads * dim | vdim]; a layer that borrows another layer's
+// keys / values points at that layer's pools.  A slot holds the list of its pages; the device copy of the table ([max_slots][pages]) is refreshed
+// at the start of a step.  Scratch buffers grow to the largest step seen and are then reused (no allocation in a steady state).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "kr_engine_internal.h"
+#include "kr_sampler.h"
+#include "kr_serve_ops.h"
+
+namespace {
+struct SvLayer {
+    kr_serve_layer d{};
+    DevBuf norm_w, norm_b, qkv, o, sink, gu, down, router, egu, edown, sgu, sdown, kpool, vpool;
+    int rope_id = 0, n_qkv = 0;
+    std::vector<char> have;      // per role (expert roles: one flag per expert)
+    int have_eg = 0, have_eu = 0, have_ed = 0;
+    std::vector<char> eg, eu, ed;
+};
+struct SvRope { int dims; double base, factor; DevBuf inv_freq; DevBuf cs; };
+struct SvSlot { bool live = false; int len = 0; std::vector<int> pages; };
+}  // namespace
+
+struct kr_serve {
+    int device = 0;
+    kr_serve_config c{};
+    bool f32 = false, finalized = false;
+    size_t esz = 2;
+    hipStream_t st = nullptr;
+    std::vector<SvLayer> L;
+    std::vector<SvRope> ropes;
+    DevBuf embed, head, fnorm_w, fnorm_b;
+    bool have_embed = false, have_head = false, have_fw = false, have_fb = false;
+    // cache
+    int n_pages = 0;
+    std::vector<int> free_pages;
+    std::vector<SvSlot> slots;
+    DevBuf page_table;
+    std::vector<int> h_table;
+    // step scratch
+    DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, moe_i, hw, logits, amax;
+    void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
+    int last_want = 0;
+    // capture / profile
+    bool capture = false; DevBuf cap; int cap_T = 0;
+    bool prof = false; double prof_ms[8] = {0}; hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // sampler scratch
+    DevBuf s_keys, s_sorted, s_temp, s_probs, s_rng, s_tok, s_seen, s_row;
+    size_t weight_bytes = 0;
+};
+
+namespace {
+uint16_t f32_to_bf16_host(float f) {
+    uint32_t b; std::memcpy(&b, &f, 4);
+    if ((b & 0x7F800000u) == 0x7F800000u && (b & 0x7FFFFFu)) return (uint16_t)((b >> 16) | 0x40);
+    b += 0x7FFFu + ((b >> 16) & 1u);
+    return (uint16_t)(b >> 16);
+}
+float bf16_to_f32_host(uint16_t v) { uint32_t b = (uint32_t)v << 16; float f; std::memcpy(&f, &b, 4); return f; }
+
+// host [n] of src_dtype -> device at dst + offset elements, as f32 (to_f32) or in the store's type
+int upload(kr_serve* s, DevBuf& dst, size_t total_elems, size_t offset_elems, const void* host, int src_dtype, size_t n, bool to_f32) {
+    const size_t esz = to_f32 ? 4 : s->esz;
+    if (!dst.p) {
+        if (dst.ensure(total_elems * esz)) return kr_fail(KR_ERR_HIP, "hipMalloc of %zu bytes failed", total_elems * esz);
+        s->weight_bytes += total_elems * esz;
+    }
+    if ((offset_elems + n) * esz > dst.bytes) return kr_fail(KR_ERR_VALUE, "tensor does not fit its slot");
+    const bool want_f32 = to_f32 || s->f32;
+    std::vector<char> tmp;
+    const void* src = host;
+    if (want_f32 && src_dtype == KR_SERVE_BF16) {
+        tmp.resize(n * 4); float* o = (float*)tmp.data(); const uint16_t* i = (const uint16_t*)host;
+        for (size_t k = 0; k < n; k++) o[k] = bf16_to_f32_host(i[k]);
+        src = tmp.data();
+    } else if (!want_f32 && src_dtype == KR_SERVE_F32) {
+        tmp.resize(n * 2); uint16_t* o = (uint16_t*)tmp.data(); const float* i = (const float*)host;
+        for (size_t k = 0; k < n; k++) o[k] = f32_to_bf16_host(i[k]);
+        src = tmp.data();
+    }
+    KR_HIP(hipMemcpy((char*)dst.p + offset_elems * esz, src, n * esz, hipMemcpyHostToDevice));
+    return KR_OK;
+}
+
+int check_layer(const kr_serve_config& c, const kr_serve_layer* all, int i) {
+    const kr_serve_layer& d = all[i];
+    if (d.heads < 1 || d.kv_heads < 1 || d.heads % d.kv_heads) return kr_fail(KR_ERR_VALUE, "layer %d: heads %d / kv_heads %d", i, d.heads, d.kv_heads);
+    if (d.dim < 1 || d.vdim < 1 || d.vdim > 512) return kr_fail(KR_ERR_VALUE, "layer %d: head sizes %d / %d (value size at most 512)", i, d.dim, d.vdim);
+    if (d.rot_dims < 0 || d.rot_dims > d.dim || (d.rot_dims & 1)) return kr_fail(KR_ERR_VALUE, "layer %d: rot_dims %d of %d", i, d.rot_dims, d.dim);
+    if (d.rot_dims && (!(d.rot_base > 0.0) || !(d.rot_factor > 0.0))) return kr_fail(KR_ERR_VALUE, "layer %d: rotation base / factor", i);
+    if (d.window < 0) return kr_fail(KR_ERR_VALUE, "layer %d: window %d", i, d.window);
+    if (d.kv_from >= 0) {
+        if (d.kv_from >= i) return kr_fail(KR_ERR_VALUE, "layer %d: kv_from %d is not an earlier layer", i, d.kv_from);
+        const kr_serve_layer& o = all[d.kv_from];
+        if (o.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d: kv_from %d has no cache of its own", i, d.kv_from);
+        if (o.kv_heads != d.kv_heads || o.dim != d.dim || o.vdim != d.vdim)
+            return kr_fail(KR_ERR_VALUE, "layer %d: key / value heads differ from layer %d", i, d.kv_from);
+    }
+    if (d.mlp_kind == KR_SERVE_MLP_DENSE && d.ff < 1) return kr_fail(KR_ERR_VALUE, "layer %d: ff %d", i, d.ff);
+    if (d.mlp_kind == KR_SERVE_MLP_MOE) {
+        if (d.experts < 1 || d.top < 1 || d.groups < 1 || d.keep < 1 || d.keep > d.groups || d.experts % d.groups || d.expert_ff < 1)
+            return kr_fail(KR_ERR_VALUE, "layer %d: router sizes (experts %d, top %d, groups %d, keep %d)", i, d.experts, d.top, d.groups, d.keep);
+        if (d.top > d.keep * (d.experts / d.groups)) return kr_fail(KR_ERR_VALUE, "layer %d: top %d exceeds the experts of %d groups", i, d.top, d.keep);
+        if (d.experts > 8192) return kr_fail(KR_ERR_VALUE, "layer %d: %d experts", i, d.experts);
+    } else if (d.mlp_kind != KR_SERVE_MLP_NONE && d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d: mlp kind %d", i, d.mlp_kind);
+    (void)c;
+    return KR_OK;
+}
+
+struct Timer {       // HIP events around one kernel family when profiling is on
+    kr_serve* s; int fam;
+    Timer(kr_serve* s_, int f) : s(s_), fam(f) { if (s->prof) (void)hipEventRecord(s->ev0, s->st); }
+    ~Timer() {
+        if (!s->prof) return;
+        (void)hipEventRecord(s->ev1, s->st); (void)hipEventSynchronize(s->ev1);
+        float ms = 0; (void)hipEventElapsedTime(&ms, s->ev0, s->ev1); s->prof_ms[fam] += ms;
+    }
+};
+}  // namespace
+
+extern "C" {
+
+int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_serve_layer* layers, kr_serve** out) {
+    if (!cfg || !layers || !out) return kr_fail(KR_ERR_VALUE, "null argument");
+    if (cfg->vocab < 1 || cfg->width < 1 || cfg->n_layers < 1) return kr_fail(KR_ERR_VALUE, "vocab / width / layers");
+    if (cfg->dtype != KR_SERVE_BF16 && cfg->dtype != KR_SERVE_F32) return kr_fail(KR_ERR_VALUE, "dtype %d", cfg->dtype);
+    if (cfg->norm_kind != KR_SERVE_NORM_LAYER && cfg->norm_kind != KR_SERVE_NORM_RMS) return kr_fail(KR_ERR_VALUE, "norm kind %d", cfg->norm_kind);
+    if (cfg->max_slots < 1 || cfg->page_tokens < 1 || cfg->pool_tokens < cfg->page_tokens) return kr_fail(KR_ERR_VALUE, "slots / pages");
+    for (int i = 0; i < cfg->n_layers; i++) { const int rc = check_layer(*cfg, layers, i); if (rc) return rc; }
+    int n_dev = 0;
+    if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev <= device_ordinal) return kr_fail(KR_ERR_HIP, "no HIP device %d (the serving store has no CPU path)", device_ordinal);
+    KR_HIP(hipSetDevice(device_ordinal));
+    kr_serve* s = new kr_serve();
+    s->device = device_ordinal; s->c = *cfg; s->f32 = cfg->dtype == KR_SERVE_F32; s->esz = s->f32 ? 4 : 2;
+    if (hipStreamCreateWithFlags(&s->st, hipStreamNonBlocking) != hipSuccess) { delete s; return kr_fail(KR_ERR_HIP, "hipStreamCreate failed"); }
+    (void)hipEventCreate(&s->ev0); (void)hipEventCreate(&s->ev1);
+    s->n_pages = cfg->pool_tokens / cfg->page_tokens;
+    for (int p = s->n_pages - 1; p >= 0; p--) s->free_pages.push_back(p);     // pop_back hands out ascending pages first
+    s->slots.resize(cfg->max_slots);
+    s->h_table.assign((size_t)cfg->max_slots * s->n_pages, 0);
+    s->L.resize(cfg->n_layers);
+    for (int i = 0; i < cfg->n_layers; i++) {
+        SvLayer& l = s->L[i]; l.d = layers[i];
+        const kr_serve_layer& d = l.d;
+        l.have.assign(KR_SV_N_ROLES, 0);
+        l.n_qkv = d.heads * d.dim + (d.kv_from < 0 ? d.kv_heads * (d.dim + d.vdim) : 0);
+        if (d.mlp_kind == KR_SERVE_MLP_MOE) { l.eg.assign(d.experts, 0); l.eu.assign(d.experts, 0); l.ed.assign(d.experts, 0); }
+        if (d.rot_dims > 0) {
+            int id = -1;
+            for (size_t r = 0; r < s->ropes.size(); r++) if (s->ropes[r].dims == d.rot_dims && s->ropes[r].base == d.rot_base && s->ropes[r].factor == d.rot_factor) id = (int)r;
+            if (id < 0) {
+                s->ropes.emplace_back(); SvRope& r = s->ropes.back(); r.dims = d.rot_dims; r.base = d.rot_base; r.factor = d.rot_factor;
+                std::vector<double> f(d.rot_dims / 2);
+                for (int k = 0; k < d.rot_dims / 2; k++) f[k] = std::pow(d.rot_base, -2.0 * k / d.rot_dims) / d.rot_factor;
+                if (r.inv_freq.ensure(f.size() * 8) || hipMemcpy(r.inv_freq.p, f.data(), f.size() * 8, hipMemcpyHostToDevice) != hipSuccess) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "rope table"); }
+                id = (int)s->ropes.size() - 1;
+            }
+            l.rope_id = id;
+        }
+        if (d.kv_from < 0) {
+            const size_t kb = (size_t)s->n_pages * cfg->page_tokens * d.kv_heads * d.dim * s->esz, vb = (size_t)s->n_pages * cfg->page_tokens * d.kv_heads * d.vdim * s->esz;
+            if (l.kpool.ensure(kb) || l.vpool.ensure(vb)) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "cache pool of %zu bytes", kb + vb); }
+            (void)hipMemset(l.kpool.p, 0, kb); (void)hipMemset(l.vpool.p, 0, vb);
+        }
+    }
+    if (s->page_table.ensure(s->h_table.size() * 4)) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "page table"); }
+    *out = s;
+    return KR_OK;
+}
+
+void kr_serve_destroy(kr_serve* s) {
+    if (!s) return;
+    (void)hipSetDevice(s->device);
+    if (s->st) { (void)hipStreamSynchronize(s->st); (void)hipStreamDestroy(s->st); }
+    if (s->ev0) (void)hipEventDestroy(s->ev0);
+    if (s->ev1) (void)hipEventDestroy(s->ev1);
+    if (s->h_meta) (void)hipHostFree(s->h_meta);
+    delete s;
+}
+
+int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void* host, int src_dtype, int rows, int cols) {
+    if (!s || !host) return kr_fail(KR_ERR_VALUE, "null argument");
+    if (src_dtype != KR_SERVE_BF16 && src_dtype != KR_SERVE_F32) return kr_fail(KR_ERR_VALUE, "source dtype %d", src_dtype);
+    KR_HIP(hipSetDevice(s->device));
+    const int W = s->c.width, V = s->c.vocab;
+    const size_t n = (size_t)rows * cols;
+#define SHAPE(R_, C_) if (rows != (R_) || cols != (C_)) return kr_fail(KR_ERR_VALUE, "layer %d role %d: shape [%d, %d], expected [%d, %d]", layer, role, rows, cols, (int)(R_), (int)(C_))
+    if (layer < 0) {
+        switch (role) {
+        case KR_SV_EMBED: SHAPE(V, W); s->have_embed = true; return upload(s, s->embed, n, 0, host, src_dtype, n, false);
+        case KR_SV_HEAD: SHAPE(V, W); s->have_head = true; return upload(s, s->head, n, 0, host, src_dtype, n, false);
+        case KR_SV_FINAL_NORM_W: SHAPE(1, W); s->have_fw = true; return upload(s, s->fnorm_w, n, 0, host, src_dtype, n, true);
+        case KR_SV_FINAL_NORM_B: SHAPE(1, W); s->have_fb = true; return upload(s, s->fnorm_b, n, 0, host, src_dtype, n, true);
+        default: return kr_fail(KR_ERR_VALUE, "role %d is not a model-level tensor", role);
+        }
+    }
+    if (layer >= s->c.n_layers) return kr_fail(KR_ERR_VALUE, "layer %d of %d", layer, s->c.n_layers);
+    SvLayer& l = s->L[layer]; const kr_serve_layer& d = l.d;
+    const int nq = d.heads * d.dim, nk = d.kv_heads * d.dim, nv = d.kv_heads * d.vdim;
+    if (role < 0 || role >= KR_SV_N_ROLES) return kr_fail(KR_ERR_VALUE, "role %d", role);
+    const bool moe = d.mlp_kind == KR_SERVE_MLP_MOE;
+    int rc = KR_OK;
+    switch (role) {
+    case KR_SV_NORM_W: SHAPE(1, W); rc = upload(s, l.norm_w, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_NORM_B: SHAPE(1, W); rc = upload(s, l.norm_b, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_Q: SHAPE(nq, W); rc = upload(s, l.qkv, (size_t)l.n_qkv * W, 0, host, src_dtype, n, false); break;
+    case KR_SV_K: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its keys", layer);
+        SHAPE(nk, W); rc = upload(s, l.qkv, (size_t)l.n_qkv * W, (size_t)nq * W, host, src_dtype, n, false); break;
+    case KR_SV_V: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its values", layer);
+        SHAPE(nv, W); rc = upload(s, l.qkv, (size_t)l.n_qkv * W, (size_t)(nq + nk) * W, host, src_dtype, n, false); break;
+    case KR_SV_O: SHAPE(W, d.heads * d.vdim); rc = upload(s, l.o, n, 0, host, src_dtype, n, false); break;
+    case KR_SV_SINK: if (!d.has_sink) return kr_fail(KR_ERR_VALUE, "layer %d has no sink", layer);
+        SHAPE(1, d.heads); rc = upload(s, l.sink, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_GATE: case KR_SV_UP:
+        if (d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d has no dense feed-forward", layer);
+        SHAPE(d.ff, W); rc = upload(s, l.gu, (size_t)2 * d.ff * W, role == KR_SV_UP ? (size_t)d.ff * W : 0, host, src_dtype, n, false); break;
+    case KR_SV_DOWN:
+        if (d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d has no dense feed-forward", layer);
+        SHAPE(W, d.ff); rc = upload(s, l.down, n, 0, host, src_dtype, n, false); break;
+    case KR_SV_ROUTER: if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no router", layer);
+        SHAPE(d.experts, W); rc = upload(s, l.router, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_EXPERT_GATE: case KR_SV_EXPERT_UP: case KR_SV_EXPERT_DOWN: {
+        if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no experts", layer);
+        if (index < 0 || index >= d.experts) return kr_fail(KR_ERR_VALUE, "expert %d of %d", index, d.experts);
+        const int F = d.expert_ff;
+        if (role == KR_SV_EXPERT_DOWN) { SHAPE(W, F); rc = upload(s, l.edown, (size_t)d.experts * W * F, (size_t)index * W * F, host, src_dtype, n, false); l.ed[index] = 1; }
+        else {
+            SHAPE(F, W);
+            rc = upload(s, l.egu, (size_t)d.experts * 2 * F * W, (size_t)index * 2 * F * W + (role == KR_SV_EXPERT_UP ? (size_t)F * W : 0), host, src_dtype, n, false);
+            (role == KR_SV_EXPERT_UP ? l.eu : l.eg)[index] = 1;
+        }
+        break;
+    }
+    case KR_SV_SHARED_GATE: case KR_SV_SHARED_UP:
+        if (!moe || d.shared_ff < 1) return kr_fail(KR_ERR_VALUE, "layer %d has no shared expert", layer);
+        SHAPE(d.shared_ff, W); rc = upload(s, l.sgu, (size_t)2 * d.shared_ff * W, role == KR_SV_SHARED_UP ? (size_t)d.shared_ff * W : 0, host, src_dtype, n, false); break;
+    case KR_SV_SHARED_DOWN:
+        if (!moe || d.shared_ff < 1) return kr_fail(KR_ERR_VALUE, "layer %d has no shared expert", layer);
+        SHAPE(W, d.shared_ff); rc = upload(s, l.sdown, n, 0, host, src_dtype, n, false); break;
+    default: return kr_fail(KR_ERR_VALUE, "role %d is not a layer tensor", role);
+    }
+#undef SHAPE
+    if (rc == KR_OK) l.have[role] = 1;
+    return rc;
+}
+
+int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp) {
+    if (!s) return kr_fail(KR_ERR_VALUE, "null argument");
+    KR_HIP(hipSetDevice(s->device));
+    const int W = s->c.width, V = s->c.vocab;
+    uint64_t k = seed;
+    // storage-type matrix [n] with fan-in `in`; f32 vectors of ones (`one`) or zeros
+    auto mat = [&](DevBuf& b, size_t n, int in) -> int {
+        if (!b.p) { if (b.ensure(n * s->esz)) return 1; s->weight_bytes += n * s->esz; }
+        kr_sv_fill_uniform(b.p, s->f32, n, ++k, amp / std::sqrt((float)in), s->st); return 0;
+    };
+    auto vec = [&](DevBuf& b, size_t n, bool one) -> int {
+        if (!b.p) { if (b.ensure(n * 4)) return 1; s->weight_bytes += n * 4; }
+        std::vector<float> h(n, one ? 1.0f : 0.0f);
+        return hipMemcpy(b.p, h.data(), n * 4, hipMemcpyHostToDevice) != hipSuccess;
+    };
+    int bad = mat(s->embed, (size_t)V * W, 1) | mat(s->head, (size_t)V * W, W) | vec(s->fnorm_w, W, true) | vec(s->fnorm_b, W, false);
+    s->have_embed = s->have_head = s->have_fw = s->have_fb = true;
+    for (SvLayer& l : s->L) {
+        const kr_serve_layer& d = l.d;
+        bad |= vec(l.norm_w, W, true) | vec(l.norm_b, W, false) | mat(l.qkv, (size_t)l.n_qkv * W, W) | mat(l.o, (size_t)W * d.heads * d.vdim, d.heads * d.vdim);
+        if (d.has_sink) bad |= vec(l.sink, d.heads, false);
+        if (d.mlp_kind == KR_SERVE_MLP_DENSE) bad |= mat(l.gu, (size_t)2 * d.ff * W, W) | mat(l.down, (size_t)W * d.ff, d.ff);
+        if (d.mlp_kind == KR_SERVE_MLP_MOE) {
+            if (!l.router.p) { if (l.router.ensure((size_t)d.experts * W * 4)) bad = 1; else s->weight_bytes += (size_t)d.experts * W * 4; }
+            if (l.router.p) kr_sv_fill_uniform(l.router.p, true, (size_t)d.experts * W, ++k, amp / std::sqrt((float)W), s->st);
+            bad |= mat(l.egu, (size_t)d.experts * 2 * d.expert_ff * W, W) | mat(l.edown, (size_t)d.experts * W * d.expert_ff, d.expert_ff);
+            if (d.shared_ff > 0) bad |= mat(l.sgu, (size_t)2 * d.shared_ff * W, W) | mat(l.sdown, (size_t)W * d.shared_ff, d.shared_ff);
+            std::fill(l.eg.begin(), l.eg.end(), 1); std::fill(l.eu.begin(), l.eu.end(), 1); std::fill(l.ed.begin(), l.ed.end(), 1);
+        }
+        std::fill(l.have.begin(), l.have.end(), 1);
+    }
+    if (bad) return kr_fail(KR_ERR_HIP, "synthetic weights: allocation or copy failed");
+    KR_HIP(hipStreamSynchronize(s->st));
+    return KR_OK;
+}
+
+int kr_serve_finalize(kr_serve* s) {
+    if (!s) return kr_fail(KR_ERR_VALUE, "null argument");
+    if (!s->have_embed || !s->have_head || !s->have_fw) return kr_fail(KR_ERR_STATE, "embedding, head or final norm missing");
+    if (s->c.norm_kind == KR_SERVE_NORM_LAYER && !s->have_fb) return kr_fail(KR_ERR_STATE, "final norm bias missing");
+    for (int i = 0; i < s->c.n_layers; i++) {
+        SvLayer& l = s->L[i]; const kr_serve_layer& d = l.d;
+        std::vector<int> need = {KR_SV_NORM_W, KR_SV_Q, KR_SV_O};
+        if (s->c.norm_kind == KR_SERVE_NORM_LAYER) need.push_back(KR_SV_NORM_B);
+        if (d.kv_from < 0) { need.push_back(KR_SV_K); need.push_back(KR_SV_V); }
+        if (d.has_sink) need.push_back(KR_SV_SINK);
+        if (d.mlp_kind == KR_SERVE_MLP_DENSE) { need.push_back(KR_SV_GATE); need.push_back(KR_SV_UP); need.push_back(KR_SV_DOWN); }
+        if (d.mlp_kind == KR_SERVE_MLP_MOE) {
+            need.push_back(KR_SV_ROUTER);
+            if (d.shared_ff > 0) { need.push_back(KR_SV_SHARED_GATE); need.push_back(KR_SV_SHARED_UP); need.push_back(KR_SV_SHARED_DOWN); }
+            for (int e = 0; e < d.experts; e++) if (!l.eg[e] || !l.eu[e] || !l.ed[e]) return kr_fail(KR_ERR_STATE, "layer %d: expert %d incomplete", i, e);
+        }
+        for (int r : need) if (!l.have[r]) return kr_fail(KR_ERR_STATE, "layer %d: tensor of role %d missing", i, r);
+    }
+    s->finalized = true;
+    return KR_OK;
+}
+
+int kr_serve_admit(kr_serve* s, int* slot_out) {
+    if (!s || !slot_out) return kr_fail(KR_ERR_VALUE, "null argument");
+    for (size_t i = 0; i < s->slots.size(); i++) if (!s->slots[i].live) { s->slots[i].live = true; s->slots[i].len = 0; *slot_out = (int)i; return KR_OK; }
+    return kr_fail(KR_ERR_STATE, "all %zu request slots are live", s->slots.size());
+}
+
+int kr_serve_release(kr_serve* s, int slot) {
+    if (!s || slot < 0 || slot >= (int)s->slots.size() || !s->slots[slot].live) return kr_fail(KR_ERR_VALUE, "slot %d is not live", slot);
+    SvSlot& sl = s->slots[slot];
+    for (size_t i = sl.pages.size(); i-- > 0;) s->free_pages.push_back(sl.pages[i]);
+    sl.pages.clear(); sl.len = 0; sl.live = false;
+    return KR_OK;
+}
+
+int kr_serve_slot_len(kr_serve* s, int slot, int* len_out) {
+    if (!s || !len_out || slot < 0 || slot >= (int)s->slots.size() || !s->slots[slot].live) return kr_fail(KR_ERR_VALUE, "slot %d is not live", slot);
+    *len_out = s->slots[slot].len; return KR_OK;
+}
+int kr_serve_free_pages(kr_serve* s, int* n_out) { if (!s || !n_out) return kr_fail(KR_ERR_VALUE, "null argument"); *n_out = (int)s->free_pages.size(); return KR_OK; }
+size_t kr_serve_device_bytes(const kr_serve* s) {
+    if (!s) return 0;
+    size_t b = s->weight_bytes;
+    for (const SvLayer& l : s->L) b += l.kpool.bytes + l.vpool.bytes;
+    return b;
+}
+int kr_serve_set_capture(kr_serve* s, int enable) { if (!s) return kr_fail(KR_ERR_VALUE, "null argument"); s->capture = enable != 0; s->cap_T = 0; return KR_OK; }
+int kr_serve_read_capture(kr_serve* s, float* out_host, size_t n_floats) {
+    if (!s || !out_host) return kr_fail(KR_ERR_VALUE, "null argument");
+    const size_t have = (size_t)s->c.n_layers * s->cap_T * s->c.width;
+    if (n_floats != have) return kr_fail(KR_ERR_VALUE, "capture holds %zu floats", have);
+    KR_HIP(hipMemcpy(out_host, s->cap.p, have * 4, hipMemcpyDeviceToHost));
+    return KR_OK;
+}
+int kr_serve_set_profiling(kr_serve* s, int enable) { if (!s) return kr_fail(KR_ERR_VALUE, "null argument"); s->prof = enable != 0; for (double& m : s->prof_ms) m = 0; return KR_OK; }
+int kr_serve_get_profile(kr_serve* s, double* ms, int n) { if (!s || !ms) return kr_fail(KR_ERR_VALUE, "null argument"); for (int i = 0; i < n && i < 8; i++) ms[i] = s->prof_ms[i]; return KR_OK; }
+
+int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* counts, const int* tokens, int n_want, const int* want_rows, float* logits_out,
+                  int* argmax_out) {
+    if (!s || !slots || !counts || !tokens || n_entries < 1 || n_want < 0 || (n_want && !want_rows)) return kr_fail(KR_ERR_VALUE, "bad step arguments");
+    if (!s->finalized) return kr_fail(KR_ERR_STATE, "the store is not finalized");
+    KR_HIP(hipSetDevice(s->device));
+    const kr_serve_config& c = s->c;
+    const int W = c.width, PT = c.page_tokens;
+    // ---- admission checks and pages, before anything changes
+    long T64 = 0; int need_pages = 0;
+    for (int e = 0; e < n_entries; e++) {
+        const int sl = slots[e];
+        if (sl < 0 || sl >= c.max_slots || !s->slots[sl].live) return kr_fail(KR_ERR_VALUE, "entry %d: slot %d is not live", e, sl);
+        for (int f = 0; f < e; f++) if (slots[f] == sl) return kr_fail(KR_ERR_VALUE, "slot %d appears twice in one step", sl);
+        if (counts[e] < 1) return kr_fail(KR_ERR_VALUE, "entry %d: %d tokens", e, counts[e]);
+        const SvSlot& q = s->slots[sl];
+        need_pages += (q.len + counts[e] + PT - 1) / PT - (int)q.pages.size();
+        T64 += counts[e];
+    }
+    if (T64 > (1 << 24)) return kr_fail(KR_ERR_VALUE, "%ld tokens in one step", T64);
+    const int T = (int)T64;
+    for (int i = 0; i < T; i++) if (tokens[i] < 0 || tokens[i] >= c.vocab) return kr_fail(KR_ERR_VALUE, "token %d outside the vocabulary", tokens[i]);
+    for (int i = 0; i < n_want; i++) if (want_rows[i] < 0 || want_rows[i] >= T) return kr_fail(KR_ERR_VALUE, "wanted row %d of %d", want_rows[i], T);
+    if (need_pages > (int)s->free_pages.size()) return kr_fail(KR_ERR_STATE, "cache pool exhausted: %d pages needed, %zu free", need_pages, s->free_pages.size());
+    // ---- per-step arrays: tokens | slot | pos | want | page table
+    const size_t n_meta = (size_t)3 * T + n_want;
+    const size_t meta_bytes = (n_meta + s->h_table.size()) * 4;
+    if (meta_bytes > s->h_meta_bytes) {
+        if (s->h_meta) (void)hipHostFree(s->h_meta);
+        s->h_meta = nullptr; s->h_meta_bytes = 0;
+        KR_HIP(hipHostMalloc(&s->h_meta, meta_bytes * 2, hipHostMallocDefault));
+        s->h_meta_bytes = meta_bytes * 2;
+    }
+    int* hm = (int*)s->h_meta;
+    int* h_tok = hm; int* h_slot = hm + T; int* h_pos = hm + 2 * T; int* h_want = hm + 3 * T; int* h_tab = hm + n_meta;
+    {
+        int t = 0;
+        for (int e = 0; e < n_entries; e++) {
+            SvSlot& q = s->slots[slots[e]];
+            const int np = (q.len + counts[e] + PT - 1) / PT;
+            while ((int)q.pages.size() < np) { q.pages.push_back(s->free_pages.back()); s->free_pages.pop_back(); }
+            for (int i = 0; i < counts[e]; i++, t++) { h_tok[t] = tokens[t]; h_slot[t] = slots[e]; h_pos[t] = q.len + i; }
+            for (size_t p = 0; p < q.pages.size(); p++) s->h_table[(size_t)slots[e] * s->n_pages + p] = q.pages[p];
+            q.len += counts[e];
+        }
+        for (int i = 0; i < n_want; i++) h_want[i] = want_rows[i];
+        std::memcpy(h_tab, s->h_table.data(), s->h_table.size() * 4);
+    }
+    if (s->meta.ensure(meta_bytes)) return kr_fail(KR_ERR_HIP, "step arrays");
+    hipStream_t st = s->st;
+    KR_HIP(hipMemcpyAsync(s->meta.p, hm, meta_bytes, hipMemcpyHostToDevice, st));
+    const int* d_tok = (const int*)s->meta.p; const int* d_slot = d_tok + T; const int* d_pos = d_tok + 2 * T; const int* d_want = d_tok + 3 * T;
+    const int* d_tab = d_tok + n_meta;
+    // ---- scratch sized for this step
+    size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0; int max_E = 1;
+    for (const SvLayer& l : s->L) {
+        const kr_serve_layer& d = l.d;
+        max_qkv = std::max(max_qkv, (size_t)l.n_qkv); max_att = std::max(max_att, (size_t)d.heads * d.vdim);
+        if (d.mlp_kind == KR_SERVE_MLP_DENSE) { max_gu = std::max(max_gu, (size_t)2 * d.ff); max_y = std::max(max_y, (size_t)d.ff); }
+        if (d.mlp_kind == KR_SERVE_MLP_MOE) {
+            max_gu = std::max(max_gu, std::max((size_t)d.top * 2 * d.expert_ff, (size_t)2 * d.shared_ff));
+            max_y = std::max(max_y, std::max((size_t)d.top * d.expert_ff, (size_t)d.shared_ff));
+            max_rows = std::max(max_rows, (size_t)d.top * W); max_pairs = std::max(max_pairs, (size_t)d.top); max_E = std::max(max_E, d.experts);
+        }
+    }
+    const size_t Ts = (size_t)T;
+    if (s->x.ensure(Ts * W * 4) || s->h.ensure(Ts * W * s->esz) || s->qkv.ensure(Ts * max_qkv * 4) || s->att.ensure(Ts * max_att * s->esz) || s->mix.ensure(Ts * W * 4) ||
+        s->gu.ensure(Ts * max_gu * 4 + 16) || s->y.ensure(Ts * max_y * s->esz + 16) || s->rows.ensure(Ts * max_rows * 4 + 16) || s->ffout.ensure(Ts * W * 4) ||
+        s->ids.ensure(Ts * max_pairs * 4 + 16) || s->wts.ensure(Ts * max_pairs * 4 + 16) || s->moe_i.ensure((Ts * max_pairs * 3 + 3 * (size_t)max_E + 8) * 4) ||
+        s->hw.ensure((size_t)std::max(n_want, 1) * W * s->esz) || s->logits.ensure((size_t)std::max(n_want, 1) * c.vocab * 4) || s->amax.ensure((size_t)std::max(n_want, 1) * 4))
+        return kr_fail(KR_ERR_HIP, "step scratch for %d tokens", T);
+    for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
+    if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
+    float* x = (float*)s->x.p;
+    {
+        Timer tm(s, 7);
+        kr_sv_embed(s->embed.p, s->f32, d_tok, x, T, W, st);
+    }
+    {
+        Timer tm(s, 2);
+        for (SvRope& r : s->ropes) kr_sv_rope_table(d_pos, (const double*)r.inv_freq.p, (float2*)r.cs.p, T, r.dims / 2, st);
+    }
+    int* mi = (int*)s->moe_i.p;
+    for (int li = 0; li < c.n_layers; li++) {
+        SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
+        { Timer tm(s, 0); kr_sv_norm(x, nullptr, (const float*)l.norm_w.p, (const float*)l.norm_b.p, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, st); }
+        KrSvGemm g{};
+        g.A = s->h.p; g.lda = W; g.W = l.qkv.p; g.C = (float*)s->qkv.p; g.ldc = l.n_qkv; g.M = T; g.N = l.n_qkv; g.K = W;
+        { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+        const SvLayer& kvl = d.kv_from >= 0 ? s->L[d.kv_from] : l;
+        KrSvAttn a{};
+        a.qkv = (float*)s->qkv.p; a.ldq = l.n_qkv; a.heads = d.heads; a.kv_heads = d.kv_heads; a.dim = d.dim; a.vdim = d.vdim; a.rot_dims = d.rot_dims;
+        a.rot_interleaved = d.rot_interleaved; a.unit_norm = d.qk_unit_norm; a.own_kv = d.kv_from < 0; a.eps = c.norm_eps; a.scale = d.scale; a.window = d.window;
+        a.sink = d.has_sink ? (const float*)l.sink.p : nullptr; a.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
+        a.kpool = kvl.kpool.p; a.vpool = kvl.vpool.p; a.page_table = d_tab; a.table_ld = s->n_pages; a.slot = d_slot; a.pos = d_pos; a.page_tokens = PT; a.T = T;
+        a.out = s->att.p;
+        { Timer tm(s, 2); kr_sv_qk_prep(a, s->f32, st); }
+        { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
+        g = KrSvGemm{};
+        g.A = s->att.p; g.lda = d.heads * d.vdim; g.W = l.o.p; g.C = (float*)s->mix.p; g.ldc = W; g.M = T; g.N = W; g.K = d.heads * d.vdim;
+        { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+        const float *dense = nullptr, *shared = nullptr, *rows = nullptr; const int* pair_pos = nullptr;
+        if (d.mlp_kind == KR_SERVE_MLP_DENSE) {
+            g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.gu.p; g.C = (float*)s->gu.p; g.ldc = 2 * d.ff; g.M = T; g.N = 2 * d.ff; g.K = W;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            { Timer tm(s, 5); kr_sv_act((const float*)s->gu.p, s->y.p, s->f32, T, d.ff, d.dense_act, 0.0f, 1.0f, st); }
+            g = KrSvGemm{}; g.A = s->y.p; g.lda = d.ff; g.W = l.down.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = d.ff;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            dense = (const float*)s->ffout.p;
+        } else if (d.mlp_kind == KR_SERVE_MLP_MOE) {
+            const int E = d.experts, top = d.top, F = d.expert_ff, P = T * top;
+            int* counts_d = mi; int* seg = mi + E; int* cursor = seg + E + 1; int* src_row = cursor + E; int* row_group = src_row + P; int* pp = row_group + P;
+            {
+                Timer tm(s, 4);
+                kr_sv_router(s->h.p, s->f32, (const float*)l.router.p, T, W, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
+                kr_sv_moe_sort((const int*)s->ids.p, T, top, E, counts_d, seg, cursor, src_row, row_group, pp, st);
+            }
+            g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.egu.p; g.w_stride = (size_t)2 * F * W; g.C = (float*)s->gu.p; g.ldc = 2 * F; g.M = P; g.N = 2 * F; g.K = W;
+            g.a_rows = src_row; g.seg = seg; g.row_group = row_group; g.n_groups = E;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            { Timer tm(s, 5); kr_sv_act((const float*)s->gu.p, s->y.p, s->f32, P, F, d.expert_act, d.expert_limit, d.expert_alpha, st); }
+            g = KrSvGemm{}; g.A = s->y.p; g.lda = F; g.W = l.edown.p; g.w_stride = (size_t)W * F; g.C = (float*)s->rows.p; g.ldc = W; g.M = P; g.N = W; g.K = F;
+            g.seg = seg; g.row_group = row_group; g.n_groups = E;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            rows = (const float*)s->rows.p; pair_pos = pp;
+            if (d.shared_ff > 0) {
+                const int SF = d.shared_ff;
+                g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.sgu.p; g.C = (float*)s->gu.p; g.ldc = 2 * SF; g.M = T; g.N = 2 * SF; g.K = W;
+                { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+                { Timer tm(s, 5); kr_sv_act((const float*)s->gu.p, s->y.p, s->f32, T, SF, d.expert_act, d.shared_limit, d.expert_alpha, st); }
+                g = KrSvGemm{}; g.A = s->y.p; g.lda = SF; g.W = l.sdown.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = SF;
+                { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+                shared = (const float*)s->ffout.p;
+            }
+        }
+        { Timer tm(s, 6); kr_sv_residual(x, (const float*)s->mix.p, dense, shared, rows, pair_pos, (const float*)s->wts.p, d.top, T, W, st); }
+        if (s->capture) KR_HIP(hipMemcpyAsync((float*)s->cap.p + (size_t)li * Ts * W, x, Ts * W * 4, hipMemcpyDeviceToDevice, st));
+    }
+    s->last_want = n_want;
+    if (n_want > 0) {
+        { Timer tm(s, 0); kr_sv_norm(x, d_want, (const float*)s->fnorm_w.p, (const float*)s->fnorm_b.p, s->hw.p, s->f32, n_want, W, c.norm_eps, c.norm_kind, st); }
+        KrSvGemm g{}; g.A = s->hw.p; g.lda = W; g.W = s->head.p; g.C = (float*)s->logits.p; g.ldc = c.vocab; g.M = n_want; g.N = c.vocab; g.K = W;
+        { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+        if (argmax_out) { Timer tm(s, 7); kr_sv_argmax((const float*)s->logits.p, n_want, c.vocab, (int*)s->amax.p, st); }
+        if (logits_out) KR_HIP(hipMemcpyAsync(logits_out, s->logits.p, (size_t)n_want * c.vocab * 4, hipMemcpyDeviceToHost, st));
+        if (argmax_out) KR_HIP(hipMemcpyAsync(argmax_out, s->amax.p, (size_t)n_want * 4, hipMemcpyDeviceToHost, st));
+    }
+    KR_HIP(hipStreamSynchronize(st));
+    KR_HIP(hipGetLastError());
+    return KR_OK;
+}
+
+int kr_serve_sample(kr_serve* s, int row, float temperature, int top_k, float top_p, uint64_t rng_seed, int* token_out) {
+    if (!s || !token_out) return kr_fail(KR_ERR_VALUE, "null argument");
+    if (row < 0 || row >= s->last_want) return kr_fail(KR_ERR_VALUE, "row %d of the last step's %d", row, s->last_want);
+    KR_HIP(hipSetDevice(s->device));
+    const int V = s->c.vocab;
+    const size_t tb = kr_sampler_temp_bytes(V);
+    if (s->s_keys.ensure((size_t)V * 8) || s->s_sorted.ensure((size_t)V * 8) || s->s_temp.ensure(tb) || s->s_probs.ensure((size_t)V * 4) || s->s_rng.ensure(8) ||
+        s->s_tok.ensure(4) || s->s_seen.ensure(((size_t)V + 31) / 32 * 4) || s->s_row.ensure((size_t)V * 4))
+        return kr_fail(KR_ERR_HIP, "sampler scratch");
+    if (!(temperature > 0.0f)) return kr_fail(KR_ERR_VALUE, "temperature %g: greedy decoding reads the step's argmax", (double)temperature);
+    KR_HIP(hipMemsetAsync(s->s_seen.p, 0, ((size_t)V + 31) / 32 * 4, s->st));
+    if (rng_seed == 0) rng_seed = 0x9E3779B97F4A7C15ull;
+    KR_HIP(hipMemcpyAsync(s->s_rng.p, &rng_seed, 8, hipMemcpyHostToDevice, s->st));
+    KR_HIP(hipMemcpyAsync(s->s_row.p, (const float*)s->logits.p + (size_t)row * V, (size_t)V * 4, hipMemcpyDeviceToDevice, s->st));   // the sampler scales in place
+    if (kr_launch_sample((float*)s->s_row.p, V, temperature, top_k, top_p, 0.0f, (uint32_t*)s->s_seen.p, (uint64_t*)s->s_keys.p, (uint64_t*)s->s_sorted.p, s->s_temp.p, tb,
+                         (float*)s->s_probs.p, (uint64_t*)s->s_rng.p, (int*)s->s_tok.p, s->st))
+        return kr_fail(KR_ERR_HIP, "sampler launch failed");
+    KR_HIP(hipMemcpyAsync(token_out, s->s_tok.p, 4, hipMemcpyDeviceToHost, s->st));
+    KR_HIP(hipStreamSynchronize(s->st));
+    return KR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,276 @@
+// kr_serve_gemm.hip -- C[M, N] (f32) = A[M, K] x W[N, K]^T for the batched serving step, single matrix or grouped (one matrix per expert, the rows
+// of a group contiguous, optional row gather for A).  Three forms:
+//   * small M (decode steps): one WAVE per output column, the K range over its lanes in 16-byte reads, up to 8 rows of A against one pass over
+//     the weight row -- bound by the weight stream;
+//   * bf16, larger M: workgroup tile 128 x 128 x 32 staged through LDS, four waves of 64 x 64 on v_mfma_f32_32x32x16_bf16, f32 accumulators, the next
+//     tile's global loads in flight during the MFMAs;
+//   * f32, larger M: 64 x 64 x 16 tile, 4 x 4 outputs per thread, plain fused multiply-adds (no reduced-precision matrix mode).
+// Every shape is accepted: edges are guarded, and rows whose byte length is not a multiple of 16 take element loads.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kr_device.h"
+#include "kr_serve_ops.h"
+
+namespace {
+typedef float gv16f __attribute__((ext_vector_type(16)));
+typedef __bf16 gb8 __attribute__((ext_vector_type(8)));
+typedef uint32_t gu4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float gm_ld(const float* p) { return *p; }
+__device__ __forceinline__ float gm_ld(const uint16_t* p) { return kr_bf16_to_f32(*p); }
+
+// row tile `tile` of a grouped problem: walks the segment table; returns false past the last tile
+__device__ __forceinline__ bool gm_find_tile(const int* seg, int n_groups, int tile, int BM, int& group, int& m0, int& mend) {
+    int acc = 0;
+    for (int g = 0; g < n_groups; g++) {
+        const int lo = seg[g], hi = seg[g + 1];
+        const int nt = (hi - lo + BM - 1) / BM;
+        if (tile < acc + nt) { group = g; m0 = lo + (tile - acc) * BM; mend = hi; return true; }
+        acc += nt;
+    }
+    return false;
+}
+
+// ---------------------------------------------------------------------------------------------------------------- small M
+template <typename T, int MB>
+__global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbase) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= g.N) return;
+    int m0 = mbase, mcnt;
+    const T* W = (const T*)g.W;
+    if (g.row_group) { m0 = blockIdx.y; mcnt = 1; W += (size_t)g.row_group[m0] * g.w_stride; }
+    else mcnt = min(MB, g.M - m0);
+    const T* wr = W + (size_t)n * g.K;
+    const T* ar[MB];
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+        const int r = min(m0 + m, g.M - 1);
+        ar[m] = (const T*)g.A + (size_t)(g.a_rows ? g.a_rows[r] : r) * g.lda;
+    }
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; m++) acc[m] = 0.0f;
+    const bool vec = (g.K % VEC == 0) && (g.lda % VEC == 0) && (((uintptr_t)g.A | (uintptr_t)g.W) % 16 == 0) && (g.w_stride % VEC == 0);
+    if (vec) {
+        for (int k = lane * VEC; k < g.K; k += 64 * VEC) {
+            const gu4 wv = *reinterpret_cast<const gu4*>(wr + k);
+            float wf[VEC];
+            if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) { wf[2 * i] = __uint_as_float(wv[i] << 16); wf[2 * i + 1] = __uint_as_float(wv[i] & 0xFFFF0000u); }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) wf[i] = __uint_as_float(wv[i]);
+            }
+#pragma unroll
+            for (int m = 0; m < MB; m++) {
+                if (m < mcnt) {
+                    const gu4 av = *reinterpret_cast<const gu4*>(ar[m] + k);
+                    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            acc[m] = __builtin_fmaf(__uint_as_float(av[i] << 16), wf[2 * i], acc[m]);
+                            acc[m] = __builtin_fmaf(__uint_as_float(av[i] & 0xFFFF0000u), wf[2 * i + 1], acc[m]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc[m] = __builtin_fmaf(__uint_as_float(av[i]), wf[i], acc[m]);
+                    }
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < g.K; k += 64) {
+            const float w = gm_ld(wr + k);
+#pragma unroll
+            for (int m = 0; m < MB; m++) if (m < mcnt) acc[m] = __builtin_fmaf(gm_ld(ar[m] + k), w, acc[m]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+        float v = acc[m];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        if (lane == 0 && m < mcnt) g.C[(size_t)(m0 + m) * g.ldc + n] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------- f32 tiles
+__global__ void __launch_bounds__(256) sv_gemm_f32_kernel(const KrSvGemm g) {
+    constexpr int BM = 64, BN = 64, BK = 16;
+    __shared__ float As[BK][BM + 4], Bs[BK][BN + 4];
+    int group = 0, m0 = blockIdx.y * BM, mend = g.M;
+    if (g.seg && !gm_find_tile(g.seg, g.n_groups, blockIdx.y, BM, group, m0, mend)) return;
+    const int n0 = blockIdx.x * BN;
+    const float* A = (const float*)g.A;
+    const float* W = (const float*)g.W + (size_t)group * g.w_stride;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    // loader: thread -> (row = tid / 4, four k = (tid % 4) * 4 ..)
+    const int lr = tid >> 2, lk = (tid & 3) * 4;
+    const int am = m0 + lr;
+    const float* arow = am < mend ? A + (size_t)(g.a_rows ? g.a_rows[am] : am) * g.lda : nullptr;
+    const float* wrow = n0 + lr < g.N ? W + (size_t)(n0 + lr) * g.K : nullptr;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = 0.0f;
+    for (int k0 = 0; k0 < g.K; k0 += BK) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int k = k0 + lk + i;
+            As[lk + i][lr] = (arow && k < g.K) ? arow[k] : 0.0f;
+            Bs[lk + i][lr] = (wrow && k < g.K) ? wrow[k] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; k++) {
+            const float4 a = *reinterpret_cast<const float4*>(&As[k][ty * 4]);
+            const float4 b = *reinterpret_cast<const float4*>(&Bs[k][tx * 4]);
+            const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= mend) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int n = n0 + tx * 4 + j;
+            if (n < g.N) g.C[(size_t)m * g.ldc + n] = acc[i][j];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------- bf16 tiles on the matrix cores
+#define GM_LD 40             // LDS row: 32 bf16 + 8 pad (80 bytes: 16-byte fragment reads of consecutive rows fall into distinct bank groups)
+template <int BM>            // 128 or 64 rows per workgroup; waves 2 x 2, each (BM / 2) x 64
+__global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
+    constexpr int BN = 128, BK = 32, MBW = BM / 64;      // 32-row blocks per wave
+    constexpr int ACH = BM * 4 / 256;                    // 16-byte chunks of the A tile per thread (rows x 4 chunks over 256 threads)
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * GM_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * GM_LD];
+    int group = 0, m0 = blockIdx.y * BM, mend = g.M;
+    if (g.seg && !gm_find_tile(g.seg, g.n_groups, blockIdx.y, BM, group, m0, mend)) return;
+    const int n0 = blockIdx.x * BN;
+    const uint16_t* A = (const uint16_t*)g.A;
+    const uint16_t* W = (const uint16_t*)g.W + (size_t)group * g.w_stride;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    const int wr = wave >> 1, wc = wave & 1;
+    const bool vec = (g.K % 8 == 0) && (g.lda % 8 == 0) && (((uintptr_t)g.A | (uintptr_t)g.W) % 16 == 0) && (g.w_stride % 8 == 0);
+    const uint16_t* ap[ACH]; const uint16_t* bp[2];
+    int akc[ACH], bkc[2];
+#pragma unroll
+    for (int i = 0; i < ACH; i++) {
+        const int c = tid + i * 256, row = c >> 2;
+        akc[i] = (c & 3) * 8;
+        const int m = m0 + row;
+        ap[i] = m < mend ? A + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : nullptr;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int c = tid + i * 256, row = c >> 2;
+        bkc[i] = (c & 3) * 8;
+        bp[i] = n0 + row < g.N ? W + (size_t)(n0 + row) * g.K : nullptr;
+    }
+    auto load16 = [&](const uint16_t* p, int k) -> gu4 {
+        gu4 v = {0u, 0u, 0u, 0u};
+        if (!p) return v;
+        if (vec) { if (k < g.K) v = *reinterpret_cast<const gu4*>(p + k); return v; }
+#pragma unroll
+        for (int i = 0; i < 8; i++) if (k + i < g.K) v[i >> 1] |= (uint32_t)p[k + i] << (16 * (i & 1));
+        return v;
+    };
+    gv16f acc[MBW][2];
+#pragma unroll
+    for (int a = 0; a < MBW; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
+    gu4 ra[ACH], rb[2];
+#pragma unroll
+    for (int i = 0; i < ACH; i++) ra[i] = load16(ap[i], akc[i]);
+#pragma unroll
+    for (int i = 0; i < 2; i++) rb[i] = load16(bp[i], bkc[i]);
+    for (int k0 = 0; k0 < g.K; k0 += BK) {
+        __syncthreads();                                 // the previous tile's fragment reads are done
+#pragma unroll
+        for (int i = 0; i < ACH; i++) { const int c = tid + i * 256; *reinterpret_cast<gu4*>(&As[(c >> 2) * GM_LD + akc[i]]) = ra[i]; }
+#pragma unroll
+        for (int i = 0; i < 2; i++) { const int c = tid + i * 256; *reinterpret_cast<gu4*>(&Bs[(c >> 2) * GM_LD + bkc[i]]) = rb[i]; }
+        __syncthreads();
+        if (k0 + BK < g.K) {
+#pragma unroll
+            for (int i = 0; i < ACH; i++) ra[i] = load16(ap[i], k0 + BK + akc[i]);
+#pragma unroll
+            for (int i = 0; i < 2; i++) rb[i] = load16(bp[i], k0 + BK + bkc[i]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            gb8 af[MBW], bf[2];
+#pragma unroll
+            for (int a = 0; a < MBW; a++) af[a] = __builtin_bit_cast(gb8, *reinterpret_cast<const gu4*>(&As[(wr * (BM / 2) + a * 32 + r) * GM_LD + ks * 16 + h * 8]));
+#pragma unroll
+            for (int b = 0; b < 2; b++) bf[b] = __builtin_bit_cast(gb8, *reinterpret_cast<const gu4*>(&Bs[(wc * 64 + b * 32 + r) * GM_LD + ks * 16 + h * 8]));
+#pragma unroll
+            for (int a = 0; a < MBW; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bf[b], acc[a][b], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < MBW; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int n = n0 + wc * 64 + b * 32 + r;
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int m = m0 + wr * (BM / 2) + a * 32 + (i & 3) + 8 * (i >> 2) + 4 * h;
+                if (m < mend) g.C[(size_t)m * g.ldc + n] = acc[a][b][i];
+            }
+        }
+}
+}  // namespace
+
+void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st) {
+    if (g.M <= 0 || g.N <= 0) return;
+    const bool grouped = g.seg != nullptr;
+    // decode-sized problems: a pass over the weights per 8 rows; grouped problems take one row per workgroup row (each row has its own expert)
+    if ((!grouped && g.M <= 16) || (grouped && g.M <= 64 && g.row_group)) {
+        if (grouped) {
+            const dim3 grid((g.N + 3) / 4, g.M);
+            if (f32) hipLaunchKernelGGL((sv_gemv_kernel<float, 1>), grid, dim3(256), 0, st, g, 0);
+            else hipLaunchKernelGGL((sv_gemv_kernel<uint16_t, 1>), grid, dim3(256), 0, st, g, 0);
+        } else {
+            KrSvGemm p = g; p.row_group = nullptr;
+            for (int mb = 0; mb < g.M; mb += 8) {
+                if (f32) hipLaunchKernelGGL((sv_gemv_kernel<float, 8>), dim3((g.N + 3) / 4), dim3(256), 0, st, p, mb);
+                else hipLaunchKernelGGL((sv_gemv_kernel<uint16_t, 8>), dim3((g.N + 3) / 4), dim3(256), 0, st, p, mb);
+            }
+        }
+        return;
+    }
+    if (f32) {
+        const int tiles = grouped ? (g.M + 63) / 64 + g.n_groups : (g.M + 63) / 64;
+        hipLaunchKernelGGL(sv_gemm_f32_kernel, dim3((g.N + 63) / 64, tiles), dim3(256), 0, st, g);
+        return;
+    }
+    // grouped problems have few rows per expert: the 64-row tile wastes less of the matrix cores
+    const bool small = grouped ? (g.M / (g.n_groups > 0 ? g.n_groups : 1) < 96) : g.M <= 64;
+    if (small) {
+        const int tiles = grouped ? (g.M + 63) / 64 + g.n_groups : (g.M + 63) / 64;
+        hipLaunchKernelGGL(sv_gemm_bf16_kernel<64>, dim3((g.N + 127) / 128, tiles), dim3(256), 0, st, g);
+    } else {
+        const int tiles = grouped ? (g.M + 127) / 128 + g.n_groups : (g.M + 127) / 128;
+        hipLaunchKernelGGL(sv_gemm_bf16_kernel<128>, dim3((g.N + 127) / 128, tiles), dim3(256), 0, st, g);
+    }
+}

@@ -1,0 +1,62 @@
+// kr_serve_ops.h -- launch wrappers of the batched serving kernels (kr_serve_ops.hip, kr_serve_gemm.hip).
+//
+// One step of the serving store is a ragged batch: T tokens of several requests, each with its own cache slot and position.  Weights, GEMM inputs
+// and cache rows have the storage type of the store (bf16 or f32: `f32` flag below); positions, angles, norms, router, scores, softmax weights and
+// the residual stream are f32 in both.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+// ---- GEMM: C[M, N] (f32) = A[M, K] x W[N, K]^T, storage type bf16 (matrix cores, f32 accumulation) or f32 (plain fused multiply-adds)
+struct KrSvGemm {
+    const void* A; int lda;          // rows of K storage elements
+    const void* W; size_t w_stride;  // [N, K] row-major; grouped: matrix g at W + g * w_stride elements
+    float* C; int ldc;
+    int M, N, K;
+    const int* a_rows;               // optional: problem row r reads A row a_rows[r]
+    const int* seg;                  // grouped: [n_groups + 1] row offsets on the device (rows of group g are [seg[g], seg[g + 1])); null = one matrix
+    const int* row_group;            // grouped: [M] group of every row (the small-M form reads it)
+    int n_groups;
+};
+void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st);
+
+enum { KR_SV_NORM_LAYER = 0, KR_SV_NORM_RMS = 1 };
+enum { KR_SV_ACT_GELU_TANH = 0, KR_SV_ACT_CLAMPED_SWIGLU = 1, KR_SV_ACT_SILU = 2 };
+
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, int T, int width, hipStream_t st);
+// out[r] = norm(x[rows ? rows[r] : r]) * w (+ b): two passes over the row, f32; out in the storage type
+void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, hipStream_t st);
+// cos / sin of pos * inv_freq for every token of the step: cs[t][i] = (cos, sin), the angle formed in double
+void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, hipStream_t st);
+
+struct KrSvAttn {
+    float* qkv; int ldq;             // [T, ldq] f32: q heads, then k heads, then v heads (k / v absent when the layer borrows another layer's cache)
+    int heads, kv_heads, dim, vdim, rot_dims, rot_interleaved, unit_norm, own_kv;
+    float eps, scale;
+    int window;                      // 0 = every earlier position
+    const float* sink;               // [heads] or null
+    const float2* cs;                // rope table of the step for this layer's rotation
+    void* kpool; void* vpool;        // [pages][page_tokens][kv_heads * dim | vdim] storage type
+    const int* page_table; int table_ld;   // [slots][table_ld]
+    const int* slot; const int* pos; // per token
+    int page_tokens, T;
+    void* out;                       // [T, heads * vdim] storage type
+};
+void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st);      // rotation, unit norm, cache append
+void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed softmax with an optional sink over the paged cache
+
+// group-limited top-k router: logits in f32 from the storage-type row and the f32 gate, softmax over all experts, the best `keep` of `groups` groups
+// (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum)
+void kr_sv_router(const void* h, bool f32, const float* gate, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
+                  hipStream_t st);
+// rows of every expert: seg[E + 1], src_row[T * top] (token of sorted row), row_group[T * top], pair_pos[T * top] (sorted row of (token, slot))
+void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st);
+// gu [M, 2F] f32 (gate | up) -> y [M, F] storage type
+void kr_sv_act(const float* gu, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st);
+// x[t] += mix[t] + (dense[t] + shared[t] + sum_s wts[t][s] * rows[pair_pos[t][s]]); null terms are skipped
+void kr_sv_residual(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
+                    int width, hipStream_t st);
+void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st);
+// uniform values in [-amp, amp) from a counter hash of (seed, element); amp = 0 writes zeros
+void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, hipStream_t st);

@@ -1,0 +1,433 @@
+// kr_serve_ops.hip -- row kernels of the batched serving step (gfx950, wave64): embedding, layer / RMS norm, rotary table, query / key preparation with
+// the paged cache append, sliding-window attention with a sink over the paged cache, group-limited top-k router, expert row sort, gated activations,
+// the parallel-block residual sum, argmax.
+//
+// Every f32 reduction here is a lane / wave tree; sums written as a * b + c may be contracted (explicit __builtin_fmaf): the serving path states a
+// tolerance against an f32 restatement, not a bit pattern.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include "kr_device.h"
+#include "kr_serve_ops.h"
+
+namespace {
+__device__ __forceinline__ float sv_ld(const float* p) { return *p; }
+__device__ __forceinline__ float sv_ld(const uint16_t* p) { return kr_bf16_to_f32(*p); }
+__device__ __forceinline__ void sv_st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void sv_st(uint16_t* p, float v) { *p = kr_f32_to_bf16(v); }
+
+__device__ __forceinline__ float sv_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ float sv_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+// sum over a workgroup of NW waves; every thread receives it
+template <int NW>
+__device__ __forceinline__ float sv_block_sum(float v, float* red) {
+    v = sv_wave_sum(v);
+    if constexpr (NW == 1) return v;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) s += red[w];
+    return s;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, int width) {
+    const int t = blockIdx.x;
+    const T* row = table + (size_t)tokens[t] * width;
+    for (int c = threadIdx.x; c < width; c += 256) x[(size_t)t * width + c] = sv_ld(row + c);
+}
+
+template <typename T, int KIND>
+__global__ void __launch_bounds__(256) sv_norm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ w, const float* __restrict__ b,
+                                                      T* __restrict__ out, int width, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[r] : r) * width;
+    float mean = 0.0f;
+    if constexpr (KIND == KR_SV_NORM_LAYER) {
+        float s = 0.0f;
+        for (int c = threadIdx.x; c < width; c += 256) s += xr[c];
+        mean = sv_block_sum<4>(s, red) / (float)width;
+    }
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < width; c += 256) { const float d = xr[c] - mean; q = __builtin_fmaf(d, d, q); }
+    const float var = sv_block_sum<4>(q, red) / (float)width;
+    const float inv = 1.0f / sqrtf(var + eps);
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float v = (xr[c] - mean) * inv * w[c];
+        if (b) v += b[c];
+        sv_st(out + (size_t)r * width + c, v);
+    }
+}
+
+__global__ void sv_rope_table_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq, float2* __restrict__ cs, int T, int half) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= T * half) return;
+    const int t = i / half, j = i - t * half;
+    const double a = (double)pos[t] * inv_freq[j];
+    cs[i] = make_float2((float)cos(a), (float)sin(a));
+}
+
+// one wave per (token, head): the head vector is staged in LDS, rotated and normed there; q heads are written back in place, k heads go to the
+// cache page of (slot, position), v heads are copied there
+template <typename T>
+__global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
+    extern __shared__ float hv[];            // [dim]
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int H = a.heads, G = a.kv_heads;
+    const int p = a.pos[t], sl = a.slot[t];
+    float* row = a.qkv + (size_t)t * a.ldq;
+    size_t prow = 0;
+    if (hh >= H) {
+        const size_t page = (size_t)a.page_table[(size_t)sl * a.table_ld + p / a.page_tokens];
+        prow = page * a.page_tokens + (p % a.page_tokens);
+    }
+    if (hh >= H + G) {                       // value head: copy
+        const int g = hh - H - G;
+        const float* v = row + (size_t)H * a.dim + (size_t)G * a.dim + (size_t)g * a.vdim;
+        T* dst = (T*)a.vpool + (prow * G + g) * a.vdim;
+        for (int d = lane; d < a.vdim; d += 64) sv_st(dst + d, v[d]);
+        return;
+    }
+    float* v = row + (size_t)hh * a.dim;
+    for (int d = lane; d < a.dim; d += 64) hv[d] = v[d];
+    __syncthreads();
+    const int half = a.rot_dims / 2;
+    const float2* cs = a.cs + (size_t)t * half;
+    float ss = 0.0f;
+    for (int i = lane; i < half; i += 64) {  // a lane owns whole rotation pairs; the tail past rot_dims passes unchanged
+        const int i0 = a.rot_interleaved ? 2 * i : i, i1 = a.rot_interleaved ? 2 * i + 1 : i + half;
+        const float u = hv[i0], w = hv[i1];
+        const float2 c = cs[i];
+        const float r0 = u * c.x - w * c.y, r1 = w * c.x + u * c.y;
+        hv[i0] = r0; hv[i1] = r1;
+        ss = __builtin_fmaf(r0, r0, ss); ss = __builtin_fmaf(r1, r1, ss);
+    }
+    for (int d = a.rot_dims + lane; d < a.dim; d += 64) ss = __builtin_fmaf(hv[d], hv[d], ss);
+    ss = sv_wave_sum(ss);
+    const float inv = a.unit_norm ? 1.0f / sqrtf(ss / (float)a.dim + a.eps) : 1.0f;
+    __syncthreads();
+    if (hh < H) {
+        for (int d = lane; d < a.dim; d += 64) v[d] = hv[d] * inv;
+    } else {
+        const int g = hh - H;
+        T* dst = (T*)a.kpool + (prow * G + g) * a.dim;
+        for (int d = lane; d < a.dim; d += 64) sv_st(dst + d, hv[d] * inv);
+    }
+}
+
+// One wave per (token, query head).  Keys [max(0, p - window + 1), p] of the token's slot are walked 64 at a time: lane j scores key j (f32 dot over dim),
+// the running maximum / denominator are updated (online softmax), and the lanes then own value columns for p.v.  The sink joins the denominator once.
+#define SV_MAX_VD 8      // value columns per lane: vdim <= 512
+template <typename T>
+__global__ void __launch_bounds__(64) sv_attn_kernel(const KrSvAttn a) {
+    extern __shared__ float lds[];           // q[dim] | p[64]
+    float* qs = lds; float* ps = lds + a.dim;
+    __shared__ size_t krow[64];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int G = a.kv_heads, g = h / (a.heads / G);
+    const int p = a.pos[t], sl = a.slot[t];
+    const int* table = a.page_table + (size_t)sl * a.table_ld;
+    const float* q = a.qkv + (size_t)t * a.ldq + (size_t)h * a.dim;
+    for (int d = lane; d < a.dim; d += 64) qs[d] = q[d];
+    __syncthreads();
+    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    float m = -INFINITY, l = 0.0f;
+    float acc[SV_MAX_VD];
+#pragma unroll
+    for (int i = 0; i < SV_MAX_VD; i++) acc[i] = 0.0f;
+    const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
+    for (int j0 = lo; j0 <= p; j0 += 64) {
+        const int j = j0 + lane;
+        float s = -INFINITY;
+        size_t prow = 0;
+        if (j <= p) {
+            prow = (size_t)table[j / a.page_tokens] * a.page_tokens + (j % a.page_tokens);
+            const T* k = kp + (prow * G + g) * a.dim;
+            float d0 = 0.0f;
+            for (int d = 0; d < a.dim; d++) d0 = __builtin_fmaf(qs[d], sv_ld(k + d), d0);
+            s = d0 * a.scale;
+        }
+        const float mn = fmaxf(m, sv_wave_max(s));
+        const float alpha = expf(m - mn);      // m = -inf on the first block: exp(-inf) = 0
+        const float pj = j <= p ? expf(s - mn) : 0.0f;
+        l = l * alpha + sv_wave_sum(pj);
+        m = mn;
+        __syncthreads();
+        ps[lane] = pj; krow[lane] = prow;
+        __syncthreads();
+        const int nk = min(64, p - j0 + 1);
+#pragma unroll
+        for (int i = 0; i < SV_MAX_VD; i++) {
+            const int d = lane + 64 * i;
+            if (d < a.vdim) {
+                float s2 = 0.0f;
+                for (int jj = 0; jj < nk; jj++) s2 = __builtin_fmaf(ps[jj], sv_ld(vp + (krow[jj] * G + g) * a.vdim + d), s2);
+                acc[i] = acc[i] * alpha + s2;
+            }
+        }
+    }
+    if (a.sink) {
+        const float sk = a.sink[h];
+        const float mn = fmaxf(m, sk);
+        const float alpha = expf(m - mn);
+        l = l * alpha + expf(sk - mn);
+#pragma unroll
+        for (int i = 0; i < SV_MAX_VD; i++) acc[i] *= alpha;
+    }
+    const float inv = 1.0f / l;
+    T* o = (T*)a.out + ((size_t)t * a.heads + h) * a.vdim;
+#pragma unroll
+    for (int i = 0; i < SV_MAX_VD; i++) {
+        const int d = lane + 64 * i;
+        if (d < a.vdim) sv_st(o + d, acc[i] * inv);
+    }
+}
+
+// one wave per token; logits / scores of the E experts live in LDS
+template <typename T>
+__global__ void __launch_bounds__(64) sv_router_kernel(const T* __restrict__ h, const float* __restrict__ gate, int width, int E, int top, int groups, int keep,
+                                                       int renorm, int* __restrict__ ids, float* __restrict__ wts) {
+    extern __shared__ float lds[];           // s[E] | gscore[groups] | allowed flags as floats [groups]
+    float* s = lds; float* gs = lds + E; float* gok = gs + groups;
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const T* x = h + (size_t)t * width;
+    for (int e = 0; e < E; e++) {
+        const float* ge = gate + (size_t)e * width;
+        float z = 0.0f;
+        for (int c = lane; c < width; c += 64) z = __builtin_fmaf(sv_ld(x + c), ge[c], z);
+        z = sv_wave_sum(z);
+        if (lane == 0) s[e] = z;
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+    mx = sv_wave_max(mx);
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) { const float v = expf(s[e] - mx); s[e] = v; sum += v; }
+    __syncthreads();
+    sum = sv_wave_sum(sum);
+    const float inv = 1.0f / sum;
+    for (int e = lane; e < E; e += 64) s[e] *= inv;
+    __syncthreads();
+    const int per = E / groups;
+    for (int gi = lane; gi < groups; gi += 64) {
+        float v = -INFINITY;
+        for (int e = gi * per; e < (gi + 1) * per; e++) v = fmaxf(v, s[e]);
+        gs[gi] = v; gok[gi] = groups == keep ? 1.0f : 0.0f;
+    }
+    __syncthreads();
+    if (keep < groups) {
+        for (int r = 0; r < keep; r++) {         // r-th best group: largest score, lowest index among equals
+            float bv = -INFINITY; int bi = 0x7fffffff;
+            for (int gi = lane; gi < groups; gi += 64) if (gok[gi] == 0.0f && (gs[gi] > bv || (gs[gi] == bv && gi < bi))) { bv = gs[gi]; bi = gi; }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(bv, o); const int oi = __shfl_xor(bi, o);
+                if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+            }
+            __syncthreads();
+            if (lane == 0 && bi != 0x7fffffff) gok[bi] = 1.0f;
+            __syncthreads();
+        }
+    }
+    float wsum = 0.0f;
+    for (int r = 0; r < top; r++) {
+        float bv = -INFINITY; int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float v = s[e];
+            if (v >= 0.0f && gok[e / per] != 0.0f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }      // a taken expert is marked by a negative score
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o); const int oi = __shfl_xor(bi, o);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        __syncthreads();
+        if (bi == 0x7fffffff) { bi = 0; bv = 0.0f; }      // fewer allowed experts than `top` (refused on the host): a zero-weight slot
+        else if (lane == 0) s[bi] = -1.0f;
+        if (lane == 0) { ids[(size_t)t * top + r] = bi; wts[(size_t)t * top + r] = bv; }
+        wsum += bv;
+        __syncthreads();
+    }
+    if (renorm) {
+        const float rinv = 1.0f / wsum;
+        for (int r = lane; r < top; r += 64) wts[(size_t)t * top + r] *= rinv;
+    }
+}
+
+__global__ void sv_fill_int_kernel(int* p, int n, int v) { const int i = blockIdx.x * blockDim.x + threadIdx.x; if (i < n) p[i] = v; }
+__global__ void sv_moe_count_kernel(const int* __restrict__ ids, int n, int* __restrict__ counts) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) atomicAdd(&counts[ids[i]], 1);
+}
+__global__ void sv_moe_scan_kernel(const int* __restrict__ counts, int E, int* __restrict__ seg, int* __restrict__ cursor) {
+    if (threadIdx.x == 0) {
+        int o = 0;
+        for (int e = 0; e < E; e++) { seg[e] = o; cursor[e] = 0; o += counts[e]; }
+        seg[E] = o;
+    }
+}
+__global__ void sv_moe_fill_kernel(const int* __restrict__ ids, int n, int top, const int* __restrict__ seg, int* __restrict__ cursor, int* __restrict__ src_row,
+                                   int* __restrict__ row_group, int* __restrict__ pair_pos) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int e = ids[i];
+    const int pos = seg[e] + atomicAdd(&cursor[e], 1);
+    src_row[pos] = i / top; row_group[pos] = e; pair_pos[i] = pos;
+}
+
+template <typename T>
+__global__ void sv_act_kernel(const float* __restrict__ gu, T* __restrict__ y, int M, int F, int kind, float limit, float alpha) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)M * F) return;
+    const size_t r = i / F; const int c = (int)(i - r * F);
+    float g = gu[r * 2 * F + c], u = gu[r * 2 * F + F + c], v;
+    if (kind == KR_SV_ACT_GELU_TANH) {
+        const float in = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+        v = 0.5f * g * (1.0f + tanhf(in)) * u;
+    } else if (kind == KR_SV_ACT_CLAMPED_SWIGLU) {
+        g = fminf(g, limit); u = fminf(fmaxf(u, -limit), limit);
+        v = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    } else {
+        v = g / (1.0f + expf(-g)) * u;
+    }
+    sv_st(y + i, v);
+}
+
+__global__ void sv_residual_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ dense, const float* __restrict__ shared,
+                                   const float* __restrict__ rows, const int* __restrict__ pair_pos, const float* __restrict__ wts, int top, int T, int width) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * width) return;
+    const size_t t = i / width; const int c = (int)(i - t * width);
+    float ff = 0.0f; bool any = false;
+    if (rows) {
+        for (int s = 0; s < top; s++) ff = __builtin_fmaf(wts[t * top + s], rows[(size_t)pair_pos[t * top + s] * width + c], ff);
+        any = true;
+    }
+    if (shared) { ff = any ? ff + shared[i] : shared[i]; any = true; }
+    if (dense) { ff = any ? ff + dense[i] : dense[i]; any = true; }
+    float d = mix ? mix[i] : 0.0f;
+    if (any) d = mix ? d + ff : ff;
+    x[i] += d;
+}
+
+__global__ void __launch_bounds__(256) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
+    __shared__ float bv[4]; __shared__ int bi[4];
+    const float* row = logits + (size_t)blockIdx.x * vocab;
+    float v = -INFINITY; int idx = 0x7fffffff;
+    for (int c = threadIdx.x; c < vocab; c += 256) { const float x = row[c]; if (x > v || (x == v && c < idx)) { v = x; idx = c; } }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o); const int oi = __shfl_xor(idx, o);
+        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = v; bi[threadIdx.x >> 6] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) if (bv[w] > v || (bv[w] == v && bi[w] < idx)) { v = bv[w]; idx = bi[w]; }
+        out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    }
+}
+template <typename T>
+__global__ void sv_fill_uniform_kernel(T* __restrict__ p, size_t n, uint64_t seed, float amp) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (i + 1);      // splitmix64 of the element index
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull; z = (z ^ (z >> 27)) * 0x94D049BB133111EBull; z ^= z >> 31;
+    const float u = (float)(z >> 40) * (1.0f / 16777216.0f);  // [0, 1)
+    sv_st(p + i, (2.0f * u - 1.0f) * amp);
+}
+}  // namespace
+
+void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, hipStream_t st) {
+    if (n == 0) return;
+    const dim3 grid((unsigned)((n + 255) / 256));
+    if (f32) hipLaunchKernelGGL(sv_fill_uniform_kernel<float>, grid, dim3(256), 0, st, (float*)p, n, seed, amp);
+    else hipLaunchKernelGGL(sv_fill_uniform_kernel<uint16_t>, grid, dim3(256), 0, st, (uint16_t*)p, n, seed, amp);
+}
+
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, int T, int width, hipStream_t st) {
+    if (T <= 0) return;
+    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, width);
+    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, width);
+}
+
+void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, hipStream_t st) {
+    if (R <= 0) return;
+#define SV_NORM(T_, K_) hipLaunchKernelGGL((sv_norm_kernel<T_, K_>), dim3(R), dim3(256), 0, st, x, rows, w, b, (T_*)out, width, eps)
+    if (kind == KR_SV_NORM_LAYER) { if (out_f32) SV_NORM(float, KR_SV_NORM_LAYER); else SV_NORM(uint16_t, KR_SV_NORM_LAYER); }
+    else { if (out_f32) SV_NORM(float, KR_SV_NORM_RMS); else SV_NORM(uint16_t, KR_SV_NORM_RMS); }
+#undef SV_NORM
+}
+
+void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, hipStream_t st) {
+    const int n = T * half;
+    if (n <= 0) return;
+    hipLaunchKernelGGL(sv_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, st, pos, inv_freq, cs, T, half);
+}
+
+void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st) {
+    if (a.T <= 0) return;
+    const dim3 grid(a.T, a.heads + (a.own_kv ? 2 * a.kv_heads : 0));
+    const size_t lds = (size_t)a.dim * sizeof(float);
+    if (f32) hipLaunchKernelGGL(sv_qk_prep_kernel<float>, grid, dim3(64), lds, st, a);
+    else hipLaunchKernelGGL(sv_qk_prep_kernel<uint16_t>, grid, dim3(64), lds, st, a);
+}
+
+void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
+    if (a.T <= 0) return;
+    const dim3 grid(a.T, a.heads);
+    const size_t lds = (size_t)(a.dim + 64) * sizeof(float);
+    if (f32) hipLaunchKernelGGL(sv_attn_kernel<float>, grid, dim3(64), lds, st, a);
+    else hipLaunchKernelGGL(sv_attn_kernel<uint16_t>, grid, dim3(64), lds, st, a);
+}
+
+void kr_sv_router(const void* h, bool f32, const float* gate, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
+                  hipStream_t st) {
+    if (T <= 0) return;
+    const size_t lds = (size_t)(E + 2 * groups) * sizeof(float);
+    if (f32) hipLaunchKernelGGL(sv_router_kernel<float>, dim3(T), dim3(64), lds, st, (const float*)h, gate, width, E, top, groups, keep, renorm, ids, wts);
+    else hipLaunchKernelGGL(sv_router_kernel<uint16_t>, dim3(T), dim3(64), lds, st, (const uint16_t*)h, gate, width, E, top, groups, keep, renorm, ids, wts);
+}
+
+void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st) {
+    const int n = T * top;
+    if (n <= 0) return;
+    hipLaunchKernelGGL(sv_fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, st, counts, E, 0);
+    hipLaunchKernelGGL(sv_moe_count_kernel, dim3((n + 255) / 256), dim3(256), 0, st, ids, n, counts);
+    hipLaunchKernelGGL(sv_moe_scan_kernel, dim3(1), dim3(64), 0, st, counts, E, seg, cursor);
+    hipLaunchKernelGGL(sv_moe_fill_kernel, dim3((n + 255) / 256), dim3(256), 0, st, ids, n, top, seg, cursor, src_row, row_group, pair_pos);
+}
+
+void kr_sv_act(const float* gu, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st) {
+    const size_t n = (size_t)M * F;
+    if (n == 0) return;
+    const dim3 grid((unsigned)((n + 255) / 256));
+    if (f32) hipLaunchKernelGGL(sv_act_kernel<float>, grid, dim3(256), 0, st, gu, (float*)y, M, F, kind, limit, alpha);
+    else hipLaunchKernelGGL(sv_act_kernel<uint16_t>, grid, dim3(256), 0, st, gu, (uint16_t*)y, M, F, kind, limit, alpha);
+}
+
+void kr_sv_residual(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
+                    int width, hipStream_t st) {
+    const size_t n = (size_t)T * width;
+    if (n == 0) return;
+    hipLaunchKernelGGL(sv_residual_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, mix, dense, shared, rows, pair_pos, wts, top, T, width);
+}
+
+void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st) {
+    if (R <= 0) return;
+    hipLaunchKernelGGL(sv_argmax_kernel, dim3(R), dim3(256), 0, st, logits, vocab, out);
+}
