@@ -342,7 +342,117 @@ def parse():
     ap.add_argument("--flip-tokens", type=int, default=2000, help="tokens of the exact-vs-KR_DECODE_FAST router-id comparison on the N = 1 line (0 = skip)")
     ap.add_argument("--detail-file", default="", help="where the full (un-abridged) result dict goes; default gpurun_out/bench_detail.json")
     ap.add_argument("--side-configs", default="v2lite-q4,v2lite-q4k-gguf,qcn-q8,qcn-q4k-gguf,qwen3-235b-q4", help="other single-GPU BASELINE configurations measured as side legs of the N = 1 line ('' = none)")
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="instead of the default workload: the layer-described Lomutar design on the batched serving store (bf16 weights, random) at a few real-model layer "
+                         "sizes -- prompt pass and decode throughput, kernel-family times -- beside the closest model of the decode graph (GQA + softmax top-k MoE, INT4) at "
+                         "the same sizes; prints its own JSON line")
+    ap.add_argument("--arch-sizes", default="small,large", help="sizes of --arch-compare (ARCH_SIZES)")
     return ap.parse_args()
+
+
+# --arch-compare: layer shapes of real mixture-of-experts models (width, heads / kv heads, head size, experts / top, expert ff, window)
+ARCH_SIZES = {
+    "small": dict(width=2048, heads=16, kv_heads=2, dim=128, experts=64, top=6, ff=768, window=1024, layers=4, vocab=32768, prompt=4096),
+    "large": dict(width=4096, heads=64, kv_heads=4, dim=128, experts=128, top=8, ff=1536, window=2048, layers=2, vocab=32768, prompt=4096),
+}
+
+
+def arch_compare(args):
+    """Throughput of the Lomutar design (batched serving store) beside the decode graph's GQA + MoE model at equal layer sizes.  Both run random weights.
+    What differs by construction: bf16 weights (4 x the bytes of INT4-g128 per decode token) and a paged multi-request cache on one side, INT4 weights with INT16
+    activations and one request on the other; the line reports tokens / s and, per side, the achieved fraction of the bound that applies (HBM bytes for decode,
+    matrix-core flops for the prompt pass)."""
+    import numpy as np
+    import torch
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    global Q235
+    out = {"metric": "arch_compare_lomutar_vs_gqa_moe", "unit": "tok/s", "sizes": {}}
+    for name in [x for x in args.arch_sizes.split(",") if x]:
+        z = ARCH_SIZES[name]; W, H, G, D, E, k, F, L, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "experts", "top", "ff", "layers", "vocab", "prompt"))
+        res = {"shape": z}
+        # ---------------- Lomutar on the serving store
+        layers = [S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, rot_dims=D // 2, rot_base=1e6, rot_factor=2.0, qk_unit_norm=1, scale=D ** -0.5, window=z["window"], has_sink=1,
+                              mlp_kind=S.MLP_MOE, experts=E, top=k, groups=4, keep=2, expert_ff=F, expert_limit=7.0, shared_ff=F, shared_limit=7.0) for _ in range(L)]
+        spec = R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None)
+        eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+        eng.load_synthetic(seed=7, amp=1.0)
+        rng = np.random.default_rng(3)
+        toks = lambda n: [int(x) for x in rng.integers(0, V, n)]
+        w_attn = (H * D + 2 * G * D) * W + W * H * D
+        w_moe_tok = (k + 1) * 3 * W * F                      # routed + shared expert, per token
+        macs_tok = L * (w_attn + w_moe_tok)
+        def prompt_pass(profile=False):
+            eng.store.set_profiling(profile)
+            t0 = time.perf_counter(); eng.step([("p", toks(P), [P - 1])], logits=False); dt = time.perf_counter() - t0
+            fam = eng.store.profile() if profile else None
+            eng.finish("p")
+            return dt, fam
+        prompt_pass()
+        ts = sorted(prompt_pass()[0] for _ in range(3)); dt = ts[1]
+        _, fam = prompt_pass(profile=True)
+        names = ["norm", "gemm", "qk_prep+rope", "attention", "router+sort", "activation", "residual", "embed+argmax"]
+        attn_flops = L * 2.0 * 2 * H * D * sum(min(i + 1, z["window"]) for i in range(P))
+        res["lomutar_prefill"] = {"tok_s": P / dt, "ms": dt * 1e3, "tokens": P, "gemm_TFLOPs": 2.0 * P * macs_tok / dt / 1e12,
+                                  "family_ms": {n: round(v, 3) for n, v in zip(names, fam)},
+                                  "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                                  "attention_family_TFLOPs": attn_flops / (fam[3] * 1e-3) / 1e12}
+        # decode: B requests at position ~ P, one token each per step
+        for B in (1, 4):
+            for b in range(B):
+                eng.step([(("d", b), toks(P), [])], logits=False)
+            ent = lambda: [(("d", b), toks(1), [0]) for b in range(B)]
+            for _ in range(5):
+                eng.step(ent(), logits=False)
+            n = 50
+            t0 = time.perf_counter()
+            for _ in range(n):
+                eng.step(ent(), logits=False)
+            dt = (time.perf_counter() - t0) / n
+            eng.store.set_profiling(True)
+            for _ in range(10):
+                eng.step(ent(), logits=False)
+            fam = [v / 10 for v in eng.store.profile()]; eng.store.set_profiling(False)
+            experts_touched = min(E, B * k)
+            byts = 2.0 * (L * (w_attn + (experts_touched + 1) * 3 * W * F + E * W * 2) + V * W)
+            res["lomutar_decode_b%d" % B] = {"tok_s": B / dt, "ms_per_step": dt * 1e3, "weight_bytes_per_step": byts, "frac_of_hbm_peak": byts / dt / 1e9 / HBM_PEAK_GBS,
+                                             "family_ms": {n_: round(v, 4) for n_, v in zip(names, fam)},
+                                             "gemm_family_frac_of_hbm_peak": byts / (fam[1] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            for b in range(B):
+                eng.finish(("d", b))
+        del eng; gc.collect()
+        # ---------------- the decode graph's GQA + MoE model at the same sizes (INT4-g128, its own single-request cache)
+        saved = Q235
+        try:
+            Q235 = dict(hidden=W, inter=F, experts=E, topk=k, layers=L, vocab=V, nh=H, nkv=G, hd=D, kv_max_seq=P + 256, eps=1e-6)
+            eng2, st, keep = build_q235(0, 0, L, P + 320, 4, False)
+            st.set_use_graph(True)
+            kvm = Q235["kv_max_seq"]
+            for key, fast in (("gqa_moe_decode_exact", False), ("gqa_moe_decode_fast", True)):
+                st.set_attention_mode(False, decode_fast=fast); st.fill_state_synthetic(kvm, seed=1)
+                def stepper(i):
+                    st.decode_step(0, P + (i % 64))
+                for i in range(5):
+                    stepper(i)
+                torch.cuda.synchronize(); t0 = time.perf_counter()
+                for i in range(50):
+                    stepper(i)
+                torch.cuda.synchronize(); dt = (time.perf_counter() - t0) / 50
+                byts = algorithmic_bytes_q235(L, B4)["total"]
+                res[key] = {"tok_s": 1 / dt, "ms_per_step": dt * 1e3, "weight_bytes_per_step": byts, "frac_of_hbm_peak": byts / dt / 1e9 / HBM_PEAK_GBS}
+            macs = q235_gemm_macs_per_token(L)
+            for key, fast, gfast in (("gqa_moe_prefill_exact", False, False), ("gqa_moe_prefill_fast", True, True)):
+                st.set_attention_mode(fast, gemm_fast=gfast)
+                r = prefill_model(st, Q235, macs, L, P, 2, torch)
+                res[key] = {"tok_s": r["value"], "ms": r["ms"], "gemm_TFLOPs": 2.0 * P * macs / (r["ms"] * 1e-3) / 1e12}
+            del eng2, st, keep; gc.collect()
+        except Exception as ex:
+            res["gqa_moe_error"] = repr(ex)
+        finally:
+            Q235 = saved
+        out["sizes"][name] = res
+    flush_native_stdout()
+    print(json.dumps(out), flush=True)
+    return out
 
 
 def is_gqa(l):
@@ -1302,6 +1412,8 @@ def main_multi(args, torch, dist, world, rank, local_rank):
 
 def main():
     args = parse()
+    if args.arch_compare:
+        return arch_compare(args)
     import torch
     import torch.distributed as dist
 

@@ -45,7 +45,7 @@ struct kr_serve {
     DevBuf page_table;
     std::vector<int> h_table;
     // step scratch
-    DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, moe_i, hw, logits, amax;
+    DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax;
     void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
     int last_want = 0;
     // capture / profile
@@ -92,7 +92,7 @@ int upload(kr_serve* s, DevBuf& dst, size_t total_elems, size_t offset_elems, co
 int check_layer(const kr_serve_config& c, const kr_serve_layer* all, int i) {
     const kr_serve_layer& d = all[i];
     if (d.heads < 1 || d.kv_heads < 1 || d.heads % d.kv_heads) return kr_fail(KR_ERR_VALUE, "layer %d: heads %d / kv_heads %d", i, d.heads, d.kv_heads);
-    if (d.dim < 1 || d.vdim < 1 || d.vdim > 512) return kr_fail(KR_ERR_VALUE, "layer %d: head sizes %d / %d (value size at most 512)", i, d.dim, d.vdim);
+    if (d.dim < 1 || d.vdim < 1 || d.vdim > 512 || d.dim > 512) return kr_fail(KR_ERR_VALUE, "layer %d: head sizes %d / %d (at most 512)", i, d.dim, d.vdim);
     if (d.rot_dims < 0 || d.rot_dims > d.dim || (d.rot_dims & 1)) return kr_fail(KR_ERR_VALUE, "layer %d: rot_dims %d of %d", i, d.rot_dims, d.dim);
     if (d.rot_dims && (!(d.rot_base > 0.0) || !(d.rot_factor > 0.0))) return kr_fail(KR_ERR_VALUE, "layer %d: rotation base / factor", i);
     if (d.window < 0) return kr_fail(KR_ERR_VALUE, "layer %d: window %d", i, d.window);
@@ -412,7 +412,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     const size_t Ts = (size_t)T;
     if (s->x.ensure(Ts * W * 4) || s->h.ensure(Ts * W * s->esz) || s->qkv.ensure(Ts * max_qkv * 4) || s->att.ensure(Ts * max_att * s->esz) || s->mix.ensure(Ts * W * 4) ||
         s->gu.ensure(Ts * max_gu * 4 + 16) || s->y.ensure(Ts * max_y * s->esz + 16) || s->rows.ensure(Ts * max_rows * 4 + 16) || s->ffout.ensure(Ts * W * 4) ||
-        s->ids.ensure(Ts * max_pairs * 4 + 16) || s->wts.ensure(Ts * max_pairs * 4 + 16) || s->moe_i.ensure((Ts * max_pairs * 3 + 3 * (size_t)max_E + 8) * 4) ||
+        s->ids.ensure(Ts * max_pairs * 4 + 16) || s->rz.ensure(Ts * (size_t)max_E * 4 + 16) || s->wts.ensure(Ts * max_pairs * 4 + 16) || s->moe_i.ensure((Ts * max_pairs * 3 + 3 * (size_t)max_E + 8) * 4) ||
         s->hw.ensure((size_t)std::max(n_want, 1) * W * s->esz) || s->logits.ensure((size_t)std::max(n_want, 1) * c.vocab * 4) || s->amax.ensure((size_t)std::max(n_want, 1) * 4))
         return kr_fail(KR_ERR_HIP, "step scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
@@ -458,7 +458,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             int* counts_d = mi; int* seg = mi + E; int* cursor = seg + E + 1; int* src_row = cursor + E; int* row_group = src_row + P; int* pp = row_group + P;
             {
                 Timer tm(s, 4);
-                kr_sv_router(s->h.p, s->f32, (const float*)l.router.p, T, W, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
+                kr_sv_router(s->h.p, s->f32, (const float*)l.router.p, (float*)s->rz.p, T, W, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
                 kr_sv_moe_sort((const int*)s->ids.p, T, top, E, counts_d, seg, cursor, src_row, row_group, pp, st);
             }
             g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.egu.p; g.w_stride = (size_t)2 * F * W; g.C = (float*)s->gu.p; g.ldc = 2 * F; g.M = P; g.N = 2 * F; g.K = W;

@@ -48,7 +48,8 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed
 
 // group-limited top-k router: logits in f32 from the storage-type row and the f32 gate, softmax over all experts, the best `keep` of `groups` groups
 // (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum)
-void kr_sv_router(const void* h, bool f32, const float* gate, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
+// z: scratch for the logits, f32 [T, E]
+void kr_sv_router(const void* h, bool f32, const float* gate, float* z, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
                   hipStream_t st);
 // rows of every expert: seg[E + 1], src_row[T * top] (token of sorted row), row_group[T * top], pair_pos[T * top] (sorted row of (token, slot))
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st);

@@ -128,89 +128,187 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
     }
 }
 
-// One wave per (token, query head).  Keys [max(0, p - window + 1), p] of the token's slot are walked 64 at a time: lane j scores key j (f32 dot over dim),
-// the running maximum / denominator are updated (online softmax), and the lanes then own value columns for p.v.  The sink joins the denominator once.
-#define SV_MAX_VD 8      // value columns per lane: vdim <= 512
-template <typename T>
-__global__ void __launch_bounds__(64) sv_attn_kernel(const KrSvAttn a) {
-    extern __shared__ float lds[];           // q[dim] | p[64]
-    float* qs = lds; float* ps = lds + a.dim;
-    __shared__ size_t krow[64];
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int G = a.kv_heads, g = h / (a.heads / G);
+// Windowed attention with a sink over the paged cache.  One workgroup (four waves) per (token, key / value head, batch of RM query heads of that
+// head's group): a cache row is fetched once for all query heads that share it.  The visible keys [max(0, p - window + 1), p] are walked in blocks of
+// 64, block b by wave b % 4; lane j scores key j for every head (f32 dot of the pre-scaled query, held in LDS, with the 16-byte pieces of its key row),
+// the wave updates each head's running maximum / denominator (online softmax, f32) and the lanes then own value columns for p.v.  The four waves'
+// partial states are merged through LDS in wave order; the sink joins the denominator there, once.
+typedef uint32_t sv_u4 __attribute__((ext_vector_type(4)));
+template <typename T, int RM, int VC>
+__global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int VEC = 16 / sizeof(T);
+    const int G = a.kv_heads, R = a.heads / G, dim = a.dim, vdim = a.vdim;
+    const int t = blockIdx.x, g = blockIdx.y, r0 = blockIdx.z * RM, nr = min(RM, R - r0), h0 = g * R + r0;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float* qs = lds;                                       // [RM][dim]
+    float* pw = qs + RM * dim + wave * 64 * RM;            // this wave's weights [RM][64]
+    float* ml = qs + RM * dim + 4 * 64 * RM;               // [4][RM][2]
+    float* accs = ml + 4 * RM * 2;                         // [RM][vdim]
     const int p = a.pos[t], sl = a.slot[t];
     const int* table = a.page_table + (size_t)sl * a.table_ld;
-    const float* q = a.qkv + (size_t)t * a.ldq + (size_t)h * a.dim;
-    for (int d = lane; d < a.dim; d += 64) qs[d] = q[d];
+    const float* q = a.qkv + (size_t)t * a.ldq + (size_t)h0 * dim;
+    for (int i = tid; i < nr * dim; i += 256) qs[i] = q[i] * a.scale;
     __syncthreads();
     const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
-    float m = -INFINITY, l = 0.0f;
-    float acc[SV_MAX_VD];
+    float m[RM], l[RM], acc[RM][VC];
 #pragma unroll
-    for (int i = 0; i < SV_MAX_VD; i++) acc[i] = 0.0f;
+    for (int r = 0; r < RM; r++) {
+        m[r] = -INFINITY; l[r] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < VC; c++) acc[r][c] = 0.0f;
+    }
     const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
-    for (int j0 = lo; j0 <= p; j0 += 64) {
+    const bool vec = ((size_t)dim * sizeof(T)) % 16 == 0;
+    for (int j0 = lo + 64 * wave; j0 <= p; j0 += 256) {
         const int j = j0 + lane;
-        float s = -INFINITY;
-        size_t prow = 0;
-        if (j <= p) {
-            prow = (size_t)table[j / a.page_tokens] * a.page_tokens + (j % a.page_tokens);
-            const T* k = kp + (prow * G + g) * a.dim;
-            float d0 = 0.0f;
-            for (int d = 0; d < a.dim; d++) d0 = __builtin_fmaf(qs[d], sv_ld(k + d), d0);
-            s = d0 * a.scale;
-        }
-        const float mn = fmaxf(m, sv_wave_max(s));
-        const float alpha = expf(m - mn);      // m = -inf on the first block: exp(-inf) = 0
-        const float pj = j <= p ? expf(s - mn) : 0.0f;
-        l = l * alpha + sv_wave_sum(pj);
-        m = mn;
-        __syncthreads();
-        ps[lane] = pj; krow[lane] = prow;
-        __syncthreads();
-        const int nk = min(64, p - j0 + 1);
+        const bool live = j <= p;
+        int prow = 0;
+        float s[RM];
 #pragma unroll
-        for (int i = 0; i < SV_MAX_VD; i++) {
-            const int d = lane + 64 * i;
-            if (d < a.vdim) {
-                float s2 = 0.0f;
-                for (int jj = 0; jj < nk; jj++) s2 = __builtin_fmaf(ps[jj], sv_ld(vp + (krow[jj] * G + g) * a.vdim + d), s2);
-                acc[i] = acc[i] * alpha + s2;
+        for (int r = 0; r < RM; r++) s[r] = 0.0f;
+        if (live) {
+            prow = table[j / a.page_tokens] * a.page_tokens + (j % a.page_tokens);
+            const T* k = kp + ((size_t)prow * G + g) * dim;
+            if (vec) {
+                for (int d = 0; d < dim; d += VEC) {
+                    const sv_u4 kv = *reinterpret_cast<const sv_u4*>(k + d);
+                    float kf[VEC];
+                    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) { kf[2 * i] = __uint_as_float(kv[i] << 16); kf[2 * i + 1] = __uint_as_float(kv[i] & 0xFFFF0000u); }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) kf[i] = __uint_as_float(kv[i]);
+                    }
+#pragma unroll
+                    for (int r = 0; r < RM; r++) {
+                        if (r < nr) {
+                            const float4* qp = reinterpret_cast<const float4*>(qs + r * dim + d);
+#pragma unroll
+                            for (int u = 0; u < VEC / 4; u++) {
+                                const float4 qa = qp[u];
+                                s[r] = __builtin_fmaf(qa.x, kf[4 * u], s[r]); s[r] = __builtin_fmaf(qa.y, kf[4 * u + 1], s[r]);
+                                s[r] = __builtin_fmaf(qa.z, kf[4 * u + 2], s[r]); s[r] = __builtin_fmaf(qa.w, kf[4 * u + 3], s[r]);
+                            }
+                        }
+                    }
+                }
+            } else {
+                for (int d = 0; d < dim; d++) {
+                    const float kd = sv_ld(k + d);
+#pragma unroll
+                    for (int r = 0; r < RM; r++) if (r < nr) s[r] = __builtin_fmaf(qs[r * dim + d], kd, s[r]);
+                }
             }
         }
-    }
-    if (a.sink) {
-        const float sk = a.sink[h];
-        const float mn = fmaxf(m, sk);
-        const float alpha = expf(m - mn);
-        l = l * alpha + expf(sk - mn);
 #pragma unroll
-        for (int i = 0; i < SV_MAX_VD; i++) acc[i] *= alpha;
-    }
-    const float inv = 1.0f / l;
-    T* o = (T*)a.out + ((size_t)t * a.heads + h) * a.vdim;
+        for (int r = 0; r < RM; r++) {
+            if (r < nr) {
+                const float sr = live ? s[r] : -INFINITY;
+                const float mn = fmaxf(m[r], sv_wave_max(sr));
+                const float alpha = expf(m[r] - mn);           // first block of this wave: exp(-inf) = 0
+                const float pj = live ? expf(sr - mn) : 0.0f;
+                l[r] = l[r] * alpha + sv_wave_sum(pj);
+                m[r] = mn;
 #pragma unroll
-    for (int i = 0; i < SV_MAX_VD; i++) {
-        const int d = lane + 64 * i;
-        if (d < a.vdim) sv_st(o + d, acc[i] * inv);
+                for (int c = 0; c < VC; c++) acc[r][c] *= alpha;
+                pw[r * 64 + lane] = pj;
+            }
+        }
+        // the wave's own LDS writes are read back by its own lanes below: a wave executes in lock step, only the LDS counter has to drain
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int nk = min(64, p - j0 + 1);
+        for (int jj = 0; jj < nk; jj++) {
+            const int pr = __builtin_amdgcn_readlane(prow, jj);
+            const T* vr = vp + ((size_t)pr * G + g) * vdim;
+            float vv[VC];
+#pragma unroll
+            for (int c = 0; c < VC; c++) { const int d = lane + 64 * c; vv[c] = d < vdim ? sv_ld(vr + d) : 0.0f; }
+#pragma unroll
+            for (int r = 0; r < RM; r++) {
+                if (r < nr) {
+                    const float w = pw[r * 64 + jj];
+#pragma unroll
+                    for (int c = 0; c < VC; c++) acc[r][c] = __builtin_fmaf(w, vv[c], acc[r][c]);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < RM; r++) if (r < nr) { ml[(wave * RM + r) * 2] = m[r]; ml[(wave * RM + r) * 2 + 1] = l[r]; }
+    }
+    __syncthreads();
+    float f[RM];
+#pragma unroll
+    for (int r = 0; r < RM; r++) {
+        f[r] = 0.0f;
+        if (r < nr) {
+            float M = -INFINITY;
+            for (int w = 0; w < 4; w++) M = fmaxf(M, ml[(w * RM + r) * 2]);
+            if (a.sink) M = fmaxf(M, a.sink[h0 + r]);
+            f[r] = expf(m[r] - M);
+        }
+    }
+    for (int w = 0; w < 4; w++) {
+        if (wave == w) {
+#pragma unroll
+            for (int r = 0; r < RM; r++) {
+                if (r < nr) {
+#pragma unroll
+                    for (int c = 0; c < VC; c++) {
+                        const int d = lane + 64 * c;
+                        if (d < vdim) accs[r * vdim + d] = (w == 0 ? 0.0f : accs[r * vdim + d]) + acc[r][c] * f[r];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    T* o = (T*)a.out + ((size_t)t * a.heads + h0) * vdim;
+    for (int i = tid; i < nr * vdim; i += 256) {
+        const int r = i / vdim;
+        float M = -INFINITY;
+        for (int w = 0; w < 4; w++) M = fmaxf(M, ml[(w * RM + r) * 2]);
+        if (a.sink) M = fmaxf(M, a.sink[h0 + r]);
+        float L = a.sink ? expf(a.sink[h0 + r] - M) : 0.0f;
+        for (int w = 0; w < 4; w++) L += ml[(w * RM + r) * 2 + 1] * expf(ml[(w * RM + r) * 2] - M);
+        sv_st(o + i, accs[i] / L);
     }
 }
 
-// one wave per token; logits / scores of the E experts live in LDS
+// router logits: z[t][e] = h[t] . gate[e] in f32; one wave per (token, four experts), the row read once for the four
 template <typename T>
-__global__ void __launch_bounds__(64) sv_router_kernel(const T* __restrict__ h, const float* __restrict__ gate, int width, int E, int top, int groups, int keep,
-                                                       int renorm, int* __restrict__ ids, float* __restrict__ wts) {
+__global__ void __launch_bounds__(256) sv_router_logits_kernel(const T* __restrict__ h, const float* __restrict__ gate, int width, int E, float* __restrict__ z) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63, e0 = (blockIdx.y * 4 + (threadIdx.x >> 6)) * 4;
+    if (e0 >= E) return;
+    const T* x = h + (size_t)t * width;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c = lane; c < width; c += 64) {
+        const float xv = sv_ld(x + c);
+#pragma unroll
+        for (int i = 0; i < 4; i++) if (e0 + i < E) acc[i] = __builtin_fmaf(xv, gate[(size_t)(e0 + i) * width + c], acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float v = sv_wave_sum(acc[i]);
+        if (lane == 0 && e0 + i < E) z[(size_t)t * E + e0 + i] = v;
+    }
+}
+
+// selection: one wave per token; the scores of the E experts live in LDS
+__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int E, int top, int groups, int keep, int renorm, int* __restrict__ ids,
+                                                              float* __restrict__ wts) {
     extern __shared__ float lds[];           // s[E] | gscore[groups] | allowed flags as floats [groups]
     float* s = lds; float* gs = lds + E; float* gok = gs + groups;
     const int t = blockIdx.x, lane = threadIdx.x;
-    const T* x = h + (size_t)t * width;
-    for (int e = 0; e < E; e++) {
-        const float* ge = gate + (size_t)e * width;
-        float z = 0.0f;
-        for (int c = lane; c < width; c += 64) z = __builtin_fmaf(sv_ld(x + c), ge[c], z);
-        z = sv_wave_sum(z);
-        if (lane == 0) s[e] = z;
-    }
+    for (int e = lane; e < E; e += 64) s[e] = z[(size_t)t * E + e];
     __syncthreads();
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
@@ -389,18 +487,26 @@ void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st) {
 
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
-    const dim3 grid(a.T, a.heads);
-    const size_t lds = (size_t)(a.dim + 64) * sizeof(float);
-    if (f32) hipLaunchKernelGGL(sv_attn_kernel<float>, grid, dim3(64), lds, st, a);
-    else hipLaunchKernelGGL(sv_attn_kernel<uint16_t>, grid, dim3(64), lds, st, a);
+    const int R = a.heads / a.kv_heads;
+    const int vc = a.vdim <= 64 ? 1 : a.vdim <= 128 ? 2 : a.vdim <= 256 ? 4 : 8;
+    const int rm = vc <= 2 ? 16 : vc == 4 ? 8 : 4;
+    const dim3 grid(a.T, a.kv_heads, (R + rm - 1) / rm);
+    const size_t lds = ((size_t)rm * a.dim + 4 * 64 * rm + 8 * rm + (size_t)rm * a.vdim) * sizeof(float);
+#define SV_ATT(T_, RM_, VC_) hipLaunchKernelGGL((sv_attn_group_kernel<T_, RM_, VC_>), grid, dim3(256), lds, st, a)
+#define SV_ATT_T(T_) do { if (vc == 1) SV_ATT(T_, 16, 1); else if (vc == 2) SV_ATT(T_, 16, 2); else if (vc == 4) SV_ATT(T_, 8, 4); else SV_ATT(T_, 4, 8); } while (0)
+    if (f32) SV_ATT_T(float); else SV_ATT_T(uint16_t);
+#undef SV_ATT_T
+#undef SV_ATT
 }
 
-void kr_sv_router(const void* h, bool f32, const float* gate, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
+void kr_sv_router(const void* h, bool f32, const float* gate, float* z, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
                   hipStream_t st) {
     if (T <= 0) return;
+    const dim3 lgrid(T, (E + 15) / 16);
+    if (f32) hipLaunchKernelGGL(sv_router_logits_kernel<float>, lgrid, dim3(256), 0, st, (const float*)h, gate, width, E, z);
+    else hipLaunchKernelGGL(sv_router_logits_kernel<uint16_t>, lgrid, dim3(256), 0, st, (const uint16_t*)h, gate, width, E, z);
     const size_t lds = (size_t)(E + 2 * groups) * sizeof(float);
-    if (f32) hipLaunchKernelGGL(sv_router_kernel<float>, dim3(T), dim3(64), lds, st, (const float*)h, gate, width, E, top, groups, keep, renorm, ids, wts);
-    else hipLaunchKernelGGL(sv_router_kernel<uint16_t>, dim3(T), dim3(64), lds, st, (const uint16_t*)h, gate, width, E, top, groups, keep, renorm, ids, wts);
+    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, E, top, groups, keep, renorm, ids, wts);
 }
 
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st) {
