@@ -6,6 +6,7 @@
 // at the start of a step.  Scratch buffers grow to the largest step seen and are then reused (no allocation in a steady state).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <string>
@@ -45,7 +46,7 @@ struct kr_serve {
     DevBuf page_table;
     std::vector<int> h_table;
     // step scratch
-    DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax;
+    DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax, part_ml, part_acc;
     void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
     int last_want = 0;
     // capture / profile
@@ -224,8 +225,18 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     case KR_SV_DOWN:
         if (d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d has no dense feed-forward", layer);
         SHAPE(W, d.ff); rc = upload(s, l.down, n, 0, host, src_dtype, n, false); break;
-    case KR_SV_ROUTER: if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no router", layer);
-        SHAPE(d.experts, W); rc = upload(s, l.router, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_ROUTER: {
+        if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no router", layer);
+        SHAPE(d.experts, W);
+        if (s->f32) { rc = upload(s, l.router, n, 0, host, src_dtype, n, false); break; }
+        // bf16 store: gate = hi + lo, both bf16, rows [0, E) and [E, 2E) of one matrix
+        std::vector<uint16_t> hl(2 * n);
+        for (size_t k = 0; k < n; k++) {
+            const float g = src_dtype == KR_SERVE_F32 ? ((const float*)host)[k] : bf16_to_f32_host(((const uint16_t*)host)[k]);
+            hl[k] = f32_to_bf16_host(g); hl[n + k] = f32_to_bf16_host(g - bf16_to_f32_host(hl[k]));
+        }
+        rc = upload(s, l.router, 2 * n, 0, hl.data(), KR_SERVE_BF16, 2 * n, false); break;
+    }
     case KR_SV_EXPERT_GATE: case KR_SV_EXPERT_UP: case KR_SV_EXPERT_DOWN: {
         if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no experts", layer);
         if (index < 0 || index >= d.experts) return kr_fail(KR_ERR_VALUE, "expert %d of %d", index, d.experts);
@@ -274,8 +285,8 @@ int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp) {
         if (d.has_sink) bad |= vec(l.sink, d.heads, false);
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) bad |= mat(l.gu, (size_t)2 * d.ff * W, W) | mat(l.down, (size_t)W * d.ff, d.ff);
         if (d.mlp_kind == KR_SERVE_MLP_MOE) {
-            if (!l.router.p) { if (l.router.ensure((size_t)d.experts * W * 4)) bad = 1; else s->weight_bytes += (size_t)d.experts * W * 4; }
-            if (l.router.p) kr_sv_fill_uniform(l.router.p, true, (size_t)d.experts * W, ++k, amp / std::sqrt((float)W), s->st);
+            bad |= mat(l.router, (size_t)d.experts * W * (s->f32 ? 1 : 2), W);
+            if (!s->f32 && l.router.p) kr_sv_fill_uniform((uint16_t*)l.router.p + (size_t)d.experts * W, false, (size_t)d.experts * W, 0, 0.0f, s->st);   // lo rows: zero
             bad |= mat(l.egu, (size_t)d.experts * 2 * d.expert_ff * W, W) | mat(l.edown, (size_t)d.experts * W * d.expert_ff, d.expert_ff);
             if (d.shared_ff > 0) bad |= mat(l.sgu, (size_t)2 * d.shared_ff * W, W) | mat(l.sdown, (size_t)W * d.shared_ff, d.shared_ff);
             std::fill(l.eg.begin(), l.eg.end(), 1); std::fill(l.eu.begin(), l.eu.end(), 1); std::fill(l.ed.begin(), l.ed.end(), 1);
@@ -379,10 +390,12 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     }
     int* hm = (int*)s->h_meta;
     int* h_tok = hm; int* h_slot = hm + T; int* h_pos = hm + 2 * T; int* h_want = hm + 3 * T; int* h_tab = hm + n_meta;
+    int max_pos = 0;
     {
         int t = 0;
         for (int e = 0; e < n_entries; e++) {
             SvSlot& q = s->slots[slots[e]];
+            max_pos = std::max(max_pos, q.len + counts[e] - 1);
             const int np = (q.len + counts[e] + PT - 1) / PT;
             while ((int)q.pages.size() < np) { q.pages.push_back(s->free_pages.back()); s->free_pages.pop_back(); }
             for (int i = 0; i < counts[e]; i++, t++) { h_tok[t] = tokens[t]; h_slot[t] = slots[e]; h_pos[t] = q.len + i; }
@@ -412,7 +425,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     const size_t Ts = (size_t)T;
     if (s->x.ensure(Ts * W * 4) || s->h.ensure(Ts * W * s->esz) || s->qkv.ensure(Ts * max_qkv * 4) || s->att.ensure(Ts * max_att * s->esz) || s->mix.ensure(Ts * W * 4) ||
         s->gu.ensure(Ts * max_gu * 4 + 16) || s->y.ensure(Ts * max_y * s->esz + 16) || s->rows.ensure(Ts * max_rows * 4 + 16) || s->ffout.ensure(Ts * W * 4) ||
-        s->ids.ensure(Ts * max_pairs * 4 + 16) || s->rz.ensure(Ts * (size_t)max_E * 4 + 16) || s->wts.ensure(Ts * max_pairs * 4 + 16) || s->moe_i.ensure((Ts * max_pairs * 3 + 3 * (size_t)max_E + 8) * 4) ||
+        s->ids.ensure(Ts * max_pairs * 4 + 16) || s->rz.ensure(Ts * (size_t)max_E * 8 + 16) || s->wts.ensure(Ts * max_pairs * 4 + 16) || s->moe_i.ensure((Ts * max_pairs * 3 + 3 * (size_t)max_E + 8) * 4) ||
         s->hw.ensure((size_t)std::max(n_want, 1) * W * s->esz) || s->logits.ensure((size_t)std::max(n_want, 1) * c.vocab * 4) || s->amax.ensure((size_t)std::max(n_want, 1) * 4))
         return kr_fail(KR_ERR_HIP, "step scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
@@ -440,6 +453,11 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         a.sink = d.has_sink ? (const float*)l.sink.p : nullptr; a.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
         a.kpool = kvl.kpool.p; a.vpool = kvl.vpool.p; a.page_table = d_tab; a.table_ld = s->n_pages; a.slot = d_slot; a.pos = d_pos; a.page_tokens = PT; a.T = T;
         a.out = s->att.p;
+        a.nsplit = kr_sv_attention_splits(T, d.heads, d.kv_heads, d.vdim, d.window > 0 ? std::min(max_pos + 1, d.window) : max_pos + 1);
+        if (a.nsplit > 1) {
+            if (s->part_ml.ensure(Ts * d.heads * a.nsplit * 8) || s->part_acc.ensure(Ts * d.heads * a.nsplit * d.vdim * 4)) return kr_fail(KR_ERR_HIP, "attention split scratch");
+            a.part_ml = (float*)s->part_ml.p; a.part_acc = (float*)s->part_acc.p;
+        }
         { Timer tm(s, 2); kr_sv_qk_prep(a, s->f32, st); }
         { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
         g = KrSvGemm{};
@@ -458,7 +476,10 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             int* counts_d = mi; int* seg = mi + E; int* cursor = seg + E + 1; int* src_row = cursor + E; int* row_group = src_row + P; int* pp = row_group + P;
             {
                 Timer tm(s, 4);
-                kr_sv_router(s->h.p, s->f32, (const float*)l.router.p, (float*)s->rz.p, T, W, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
+                const int parts = s->f32 ? 1 : 2;
+                KrSvGemm rg{}; rg.A = s->h.p; rg.lda = W; rg.W = l.router.p; rg.C = (float*)s->rz.p; rg.ldc = parts * E; rg.M = T; rg.N = parts * E; rg.K = W;
+                kr_sv_gemm(rg, s->f32, st);
+                kr_sv_router_select((const float*)s->rz.p, parts, T, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
                 kr_sv_moe_sort((const int*)s->ids.p, T, top, E, counts_d, seg, cursor, src_row, row_group, pp, st);
             }
             g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.egu.p; g.w_stride = (size_t)2 * F * W; g.C = (float*)s->gu.p; g.ldc = 2 * F; g.M = P; g.N = 2 * F; g.K = W;

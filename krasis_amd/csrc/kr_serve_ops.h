@@ -42,15 +42,19 @@ struct KrSvAttn {
     const int* slot; const int* pos; // per token
     int page_tokens, T;
     void* out;                       // [T, heads * vdim] storage type
+    int nsplit;                      // >= 1: workgroups that share a token's keys (few tokens: more of the chip per token); > 1 needs the two buffers below
+    float* part_ml; float* part_acc; // [T][heads][nsplit][2] running (maximum, denominator), [T][heads][nsplit][vdim] unnormalised sums
 };
+// how many ways to split: fills the chip when the step has few tokens; max_visible = most keys any token of the step sees in this layer
+int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_visible);
 void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st);      // rotation, unit norm, cache append
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed softmax with an optional sink over the paged cache
 
-// group-limited top-k router: logits in f32 from the storage-type row and the f32 gate, softmax over all experts, the best `keep` of `groups` groups
-// (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum)
-// z: scratch for the logits, f32 [T, E]
-void kr_sv_router(const void* h, bool f32, const float* gate, float* z, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
-                  hipStream_t st);
+// group-limited top-k router on logits z [T, parts * E] f32 (the `parts` column blocks are added): softmax over all experts, the best `keep` of
+// `groups` groups (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum).
+// The logits come from kr_sv_gemm: an f32 store multiplies by the f32 gate; a bf16 store by the gate as two bf16 terms (hi + lo rows), which
+// carries 16 bits of the gate's mantissa through the matrix cores.
+void kr_sv_router_select(const float* z, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st);
 // rows of every expert: seg[E + 1], src_row[T * top] (token of sorted row), row_group[T * top], pair_pos[T * top] (sorted row of (token, slot))
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st);
 // gu [M, 2F] f32 (gate | up) -> y [M, F] storage type

@@ -8,6 +8,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "kr_device.h"
 #include "kr_serve_ops.h"
 
@@ -17,15 +19,16 @@ __device__ __forceinline__ float sv_ld(const uint16_t* p) { return kr_bf16_to_f3
 __device__ __forceinline__ void sv_st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void sv_st(uint16_t* p, float v) { *p = kr_f32_to_bf16(v); }
 
+// wave-wide sum / maximum, every lane receives it: four DPP steps inside each row of 16 lanes, then the four rows through scalar reads
+#define SV_DPPF(v, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), (ctrl), 0xF, 0xF, false))
+#define SV_LANE(v, i) __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), (i)))
 __device__ __forceinline__ float sv_wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
+    v += SV_DPPF(v, KR_DPP_XOR1); v += SV_DPPF(v, KR_DPP_XOR2); v += SV_DPPF(v, KR_DPP_HALF_MIRROR); v += SV_DPPF(v, KR_DPP_MIRROR);
+    return (SV_LANE(v, 0) + SV_LANE(v, 16)) + (SV_LANE(v, 32) + SV_LANE(v, 48));
 }
 __device__ __forceinline__ float sv_wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
+    v = fmaxf(v, SV_DPPF(v, KR_DPP_XOR1)); v = fmaxf(v, SV_DPPF(v, KR_DPP_XOR2)); v = fmaxf(v, SV_DPPF(v, KR_DPP_HALF_MIRROR)); v = fmaxf(v, SV_DPPF(v, KR_DPP_MIRROR));
+    return fmaxf(fmaxf(SV_LANE(v, 0), SV_LANE(v, 16)), fmaxf(SV_LANE(v, 32), SV_LANE(v, 48)));
 }
 // sum over a workgroup of NW waves; every thread receives it
 template <int NW>
@@ -139,7 +142,8 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int VEC = 16 / sizeof(T);
     const int G = a.kv_heads, R = a.heads / G, dim = a.dim, vdim = a.vdim;
-    const int t = blockIdx.x, g = blockIdx.y, r0 = blockIdx.z * RM, nr = min(RM, R - r0), h0 = g * R + r0;
+    const int sp = blockIdx.z % a.nsplit;
+    const int t = blockIdx.x, g = blockIdx.y, r0 = (blockIdx.z / a.nsplit) * RM, nr = min(RM, R - r0), h0 = g * R + r0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float* qs = lds;                                       // [RM][dim]
     float* pw = qs + RM * dim + wave * 64 * RM;            // this wave's weights [RM][64]
@@ -148,7 +152,9 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     const int p = a.pos[t], sl = a.slot[t];
     const int* table = a.page_table + (size_t)sl * a.table_ld;
     const float* q = a.qkv + (size_t)t * a.ldq + (size_t)h0 * dim;
-    for (int i = tid; i < nr * dim; i += 256) qs[i] = q[i] * a.scale;
+    // heads past the group's last one are computed on zero queries and dropped: the loops below carry no per-head branches, so the loads of a block of
+    // keys are all in flight before the first product needs them
+    for (int i = tid; i < RM * dim; i += 256) qs[i] = i < nr * dim ? q[i] * a.scale : 0.0f;
     __syncthreads();
     const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
     float m[RM], l[RM], acc[RM][VC];
@@ -160,79 +166,105 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     }
     const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
     const bool vec = ((size_t)dim * sizeof(T)) % 16 == 0;
-    for (int j0 = lo + 64 * wave; j0 <= p; j0 += 256) {
+    const int npiece = dim / VEC;
+    auto widen = [](const sv_u4& kv, float* kf) {
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) { kf[2 * i] = __uint_as_float(kv[i] << 16); kf[2 * i + 1] = __uint_as_float(kv[i] & 0xFFFF0000u); }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) kf[i] = __uint_as_float(kv[i]);
+        }
+    };
+    // blocks of 64 keys: this workgroup's share [c0, c1) of the token's blocks (all of them when the launch is not split), block c by wave (c - c0) % 4
+    const int nch = (p - lo) / 64 + 1, cps = (nch + a.nsplit - 1) / a.nsplit;
+    const int c0 = sp * cps, c1 = min(nch, c0 + cps);
+    for (int cb = c0 + wave; cb < c1; cb += 4) {
+        const int j0 = lo + 64 * cb;
         const int j = j0 + lane;
         const bool live = j <= p;
-        int prow = 0;
+        const int jc = min(j, p);                            // lanes past the last key score it again; their weight is set to 0
+        const int prow = table[jc / a.page_tokens] * a.page_tokens + (jc % a.page_tokens);
+        const T* k = kp + ((size_t)prow * G + g) * dim;
         float s[RM];
 #pragma unroll
         for (int r = 0; r < RM; r++) s[r] = 0.0f;
-        if (live) {
-            prow = table[j / a.page_tokens] * a.page_tokens + (j % a.page_tokens);
-            const T* k = kp + ((size_t)prow * G + g) * dim;
-            if (vec) {
-                for (int d = 0; d < dim; d += VEC) {
-                    const sv_u4 kv = *reinterpret_cast<const sv_u4*>(k + d);
+        if (vec) {
+            int pc = 0;
+            auto block = [&](auto PBc) {                     // PB 16-byte pieces of the key row in flight, then their products with every head's query
+                constexpr int PB = decltype(PBc)::value;
+                sv_u4 kv[PB];
+#pragma unroll
+                for (int u = 0; u < PB; u++) kv[u] = *reinterpret_cast<const sv_u4*>(k + (pc + u) * VEC);
+#pragma unroll
+                for (int u = 0; u < PB; u++) {
                     float kf[VEC];
-                    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-                        for (int i = 0; i < 4; i++) { kf[2 * i] = __uint_as_float(kv[i] << 16); kf[2 * i + 1] = __uint_as_float(kv[i] & 0xFFFF0000u); }
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < 4; i++) kf[i] = __uint_as_float(kv[i]);
-                    }
+                    widen(kv[u], kf);
 #pragma unroll
                     for (int r = 0; r < RM; r++) {
-                        if (r < nr) {
-                            const float4* qp = reinterpret_cast<const float4*>(qs + r * dim + d);
+                        const float4* qp = reinterpret_cast<const float4*>(qs + r * dim + (pc + u) * VEC);
 #pragma unroll
-                            for (int u = 0; u < VEC / 4; u++) {
-                                const float4 qa = qp[u];
-                                s[r] = __builtin_fmaf(qa.x, kf[4 * u], s[r]); s[r] = __builtin_fmaf(qa.y, kf[4 * u + 1], s[r]);
-                                s[r] = __builtin_fmaf(qa.z, kf[4 * u + 2], s[r]); s[r] = __builtin_fmaf(qa.w, kf[4 * u + 3], s[r]);
-                            }
+                        for (int v4 = 0; v4 < VEC / 4; v4++) {
+                            const float4 qa = qp[v4];
+                            s[r] = __builtin_fmaf(qa.x, kf[4 * v4], s[r]); s[r] = __builtin_fmaf(qa.y, kf[4 * v4 + 1], s[r]);
+                            s[r] = __builtin_fmaf(qa.z, kf[4 * v4 + 2], s[r]); s[r] = __builtin_fmaf(qa.w, kf[4 * v4 + 3], s[r]);
                         }
                     }
                 }
-            } else {
-                for (int d = 0; d < dim; d++) {
-                    const float kd = sv_ld(k + d);
+                pc += PB;
+            };
+            while (pc + 8 <= npiece) block(std::integral_constant<int, 8>{});
+            if (pc + 4 <= npiece) block(std::integral_constant<int, 4>{});
+            for (; pc < npiece; pc++) {
+                const sv_u4 kv = *reinterpret_cast<const sv_u4*>(k + pc * VEC);
+                float kf[VEC];
+                widen(kv, kf);
 #pragma unroll
-                    for (int r = 0; r < RM; r++) if (r < nr) s[r] = __builtin_fmaf(qs[r * dim + d], kd, s[r]);
-                }
+                for (int r = 0; r < RM; r++)
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) s[r] = __builtin_fmaf(qs[r * dim + pc * VEC + i], kf[i], s[r]);
+            }
+        } else {
+            for (int d = 0; d < dim; d++) {
+                const float kd = sv_ld(k + d);
+#pragma unroll
+                for (int r = 0; r < RM; r++) s[r] = __builtin_fmaf(qs[r * dim + d], kd, s[r]);
             }
         }
 #pragma unroll
         for (int r = 0; r < RM; r++) {
-            if (r < nr) {
-                const float sr = live ? s[r] : -INFINITY;
-                const float mn = fmaxf(m[r], sv_wave_max(sr));
-                const float alpha = expf(m[r] - mn);           // first block of this wave: exp(-inf) = 0
-                const float pj = live ? expf(sr - mn) : 0.0f;
-                l[r] = l[r] * alpha + sv_wave_sum(pj);
-                m[r] = mn;
+            const float sr = live ? s[r] : -INFINITY;
+            const float mn = fmaxf(m[r], sv_wave_max(sr));
+            const float alpha = expf(m[r] - mn);               // first block of this wave: exp(-inf) = 0
+            const float pj = live ? expf(sr - mn) : 0.0f;
+            l[r] = l[r] * alpha + sv_wave_sum(pj);
+            m[r] = mn;
 #pragma unroll
-                for (int c = 0; c < VC; c++) acc[r][c] *= alpha;
-                pw[r * 64 + lane] = pj;
-            }
+            for (int c = 0; c < VC; c++) acc[r][c] *= alpha;
+            pw[r * 64 + lane] = pj;
         }
         // the wave's own LDS writes are read back by its own lanes below: a wave executes in lock step, only the LDS counter has to drain
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int U = 16 / VC;                           // keys whose value rows are in flight together
         const int nk = min(64, p - j0 + 1);
-        for (int jj = 0; jj < nk; jj++) {
-            const int pr = __builtin_amdgcn_readlane(prow, jj);
-            const T* vr = vp + ((size_t)pr * G + g) * vdim;
-            float vv[VC];
+        for (int jb = 0; jb < nk; jb += U) {                 // keys past nk inside the last group carry weight 0 and read the last key's row
+            float vv[U][VC];
 #pragma unroll
-            for (int c = 0; c < VC; c++) { const int d = lane + 64 * c; vv[c] = d < vdim ? sv_ld(vr + d) : 0.0f; }
+            for (int u = 0; u < U; u++) {
+                const int pr = __builtin_amdgcn_readlane(prow, min(jb + u, 63));
+                const T* vr = vp + ((size_t)pr * G + g) * vdim;
+#pragma unroll
+                for (int c = 0; c < VC; c++) { const int d = lane + 64 * c; vv[u][c] = d < vdim ? sv_ld(vr + d) : 0.0f; }
+            }
 #pragma unroll
             for (int r = 0; r < RM; r++) {
-                if (r < nr) {
-                    const float w = pw[r * 64 + jj];
 #pragma unroll
-                    for (int c = 0; c < VC; c++) acc[r][c] = __builtin_fmaf(w, vv[c], acc[r][c]);
+                for (int u = 0; u < U; u++) {
+                    const float w = pw[r * 64 + min(jb + u, 63)];
+#pragma unroll
+                    for (int c = 0; c < VC; c++) acc[r][c] = __builtin_fmaf(w, vv[u][c], acc[r][c]);
                 }
             }
         }
@@ -245,6 +277,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         for (int r = 0; r < RM; r++) if (r < nr) { ml[(wave * RM + r) * 2] = m[r]; ml[(wave * RM + r) * 2 + 1] = l[r]; }
     }
     __syncthreads();
+    const bool last = a.nsplit == 1;                         // an unsplit launch finishes here: sink, normalisation, output; a split one leaves partial states
     float f[RM];
 #pragma unroll
     for (int r = 0; r < RM; r++) {
@@ -252,8 +285,8 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         if (r < nr) {
             float M = -INFINITY;
             for (int w = 0; w < 4; w++) M = fmaxf(M, ml[(w * RM + r) * 2]);
-            if (a.sink) M = fmaxf(M, a.sink[h0 + r]);
-            f[r] = expf(m[r] - M);
+            if (last && a.sink) M = fmaxf(M, a.sink[h0 + r]);
+            f[r] = m[r] == -INFINITY ? 0.0f : expf(m[r] - M);
         }
     }
     for (int w = 0; w < 4; w++) {
@@ -276,39 +309,43 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         const int r = i / vdim;
         float M = -INFINITY;
         for (int w = 0; w < 4; w++) M = fmaxf(M, ml[(w * RM + r) * 2]);
-        if (a.sink) M = fmaxf(M, a.sink[h0 + r]);
-        float L = a.sink ? expf(a.sink[h0 + r] - M) : 0.0f;
-        for (int w = 0; w < 4; w++) L += ml[(w * RM + r) * 2 + 1] * expf(ml[(w * RM + r) * 2] - M);
-        sv_st(o + i, accs[i] / L);
+        if (last && a.sink) M = fmaxf(M, a.sink[h0 + r]);
+        float L = (last && a.sink) ? expf(a.sink[h0 + r] - M) : 0.0f;
+        for (int w = 0; w < 4; w++) { const float mw = ml[(w * RM + r) * 2]; if (mw != -INFINITY) L += ml[(w * RM + r) * 2 + 1] * expf(mw - M); }
+        if (last) sv_st(o + i, accs[i] / L);
+        else {
+            const size_t slot = ((size_t)t * a.heads + h0 + r) * a.nsplit + sp;
+            a.part_acc[slot * vdim + (i - r * vdim)] = accs[i];
+            if (i == r * vdim) { a.part_ml[slot * 2] = M; a.part_ml[slot * 2 + 1] = L; }
+        }
     }
 }
 
-// router logits: z[t][e] = h[t] . gate[e] in f32; one wave per (token, four experts), the row read once for the four
+// the partial states of a split launch -> output: one wave per (token, head)
 template <typename T>
-__global__ void __launch_bounds__(256) sv_router_logits_kernel(const T* __restrict__ h, const float* __restrict__ gate, int width, int E, float* __restrict__ z) {
-    const int t = blockIdx.x, lane = threadIdx.x & 63, e0 = (blockIdx.y * 4 + (threadIdx.x >> 6)) * 4;
-    if (e0 >= E) return;
-    const T* x = h + (size_t)t * width;
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int c = lane; c < width; c += 64) {
-        const float xv = sv_ld(x + c);
-#pragma unroll
-        for (int i = 0; i < 4; i++) if (e0 + i < E) acc[i] = __builtin_fmaf(xv, gate[(size_t)(e0 + i) * width + c], acc[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float v = sv_wave_sum(acc[i]);
-        if (lane == 0 && e0 + i < E) z[(size_t)t * E + e0 + i] = v;
+__global__ void __launch_bounds__(64) sv_attn_merge_kernel(const KrSvAttn a) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const size_t base = ((size_t)t * a.heads + h) * a.nsplit;
+    float M = a.sink ? a.sink[h] : -INFINITY;
+    for (int s = 0; s < a.nsplit; s++) M = fmaxf(M, a.part_ml[(base + s) * 2]);
+    float L = a.sink ? expf(a.sink[h] - M) : 0.0f;
+    for (int s = 0; s < a.nsplit; s++) { const float ms = a.part_ml[(base + s) * 2]; if (ms != -INFINITY) L += a.part_ml[(base + s) * 2 + 1] * expf(ms - M); }
+    T* o = (T*)a.out + ((size_t)t * a.heads + h) * a.vdim;
+    for (int d = lane; d < a.vdim; d += 64) {
+        float v = 0.0f;
+        for (int s = 0; s < a.nsplit; s++) { const float ms = a.part_ml[(base + s) * 2]; if (ms != -INFINITY) v = __builtin_fmaf(a.part_acc[(base + s) * a.vdim + d], expf(ms - M), v); }
+        sv_st(o + d, v / L);
     }
 }
 
 // selection: one wave per token; the scores of the E experts live in LDS
-__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int E, int top, int groups, int keep, int renorm, int* __restrict__ ids,
-                                                              float* __restrict__ wts) {
+// z holds the logits as `parts` column blocks of E that are added (a gate stored as two bf16 terms gives two)
+__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int parts, int E, int top, int groups, int keep, int renorm,
+                                                              int* __restrict__ ids, float* __restrict__ wts) {
     extern __shared__ float lds[];           // s[E] | gscore[groups] | allowed flags as floats [groups]
     float* s = lds; float* gs = lds + E; float* gok = gs + groups;
     const int t = blockIdx.x, lane = threadIdx.x;
-    for (int e = lane; e < E; e += 64) s[e] = z[(size_t)t * E + e];
+    for (int e = lane; e < E; e += 64) { float v = z[(size_t)t * parts * E + e]; for (int q = 1; q < parts; q++) v += z[((size_t)t * parts + q) * E + e]; s[e] = v; }
     __syncthreads();
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
@@ -385,6 +422,28 @@ __global__ void sv_moe_fill_kernel(const int* __restrict__ ids, int n, int top, 
     const int e = ids[i];
     const int pos = seg[e] + atomicAdd(&cursor[e], 1);
     src_row[pos] = i / top; row_group[pos] = e; pair_pos[i] = pos;
+}
+
+// the three launches above as one workgroup, for decode-sized batches (n pairs <= 1024, E counters in LDS)
+__global__ void __launch_bounds__(256) sv_moe_sort_small_kernel(const int* __restrict__ ids, int n, int top, int E, int* __restrict__ seg, int* __restrict__ src_row,
+                                                                int* __restrict__ row_group, int* __restrict__ pair_pos) {
+    extern __shared__ int cnt[];             // counts[E] | start[E]
+    int* start = cnt + E;
+    for (int e = threadIdx.x; e < E; e += 256) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 256) atomicAdd(&cnt[ids[i]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int o = 0;
+        for (int e = 0; e < E; e++) { start[e] = o; seg[e] = o; o += cnt[e]; cnt[e] = 0; }
+        seg[E] = o;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const int e = ids[i];
+        const int pos = start[e] + atomicAdd(&cnt[e], 1);
+        src_row[pos] = i / top; row_group[pos] = e; pair_pos[i] = pos;
+    }
 }
 
 template <typename T>
@@ -485,33 +544,55 @@ void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st) {
     else hipLaunchKernelGGL(sv_qk_prep_kernel<uint16_t>, grid, dim3(64), lds, st, a);
 }
 
+int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_visible) {
+    const int R = heads / kv_heads;
+    const int vc = vdim <= 64 ? 1 : vdim <= 128 ? 2 : vdim <= 256 ? 4 : 8;
+    const int rmax = vc <= 2 ? 16 : vc == 4 ? 8 : 4;
+    int rm = 2;
+    while (rm < R && rm < rmax) rm *= 2;
+    const long blocks = (long)T * kv_heads * ((R + rm - 1) / rm);
+    const int nch = (max_visible + 63) / 64;
+    long ns = 1024 / (blocks > 0 ? blocks : 1);              // about four workgroups per compute unit
+    if (ns > (nch + 3) / 4) ns = (nch + 3) / 4;              // a workgroup keeps at least one block of keys per wave
+    return ns < 1 ? 1 : (int)ns;
+}
+
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
     const int R = a.heads / a.kv_heads;
     const int vc = a.vdim <= 64 ? 1 : a.vdim <= 128 ? 2 : a.vdim <= 256 ? 4 : 8;
-    const int rm = vc <= 2 ? 16 : vc == 4 ? 8 : 4;
-    const dim3 grid(a.T, a.kv_heads, (R + rm - 1) / rm);
+    const int rmax = vc <= 2 ? 16 : vc == 4 ? 8 : 4;       // RM * VC accumulators per lane stay within 32
+    int rm = 2;
+    while (rm < R && rm < rmax) rm *= 2;
+    const dim3 grid(a.T, a.kv_heads, ((R + rm - 1) / rm) * a.nsplit);
     const size_t lds = ((size_t)rm * a.dim + 4 * 64 * rm + 8 * rm + (size_t)rm * a.vdim) * sizeof(float);
 #define SV_ATT(T_, RM_, VC_) hipLaunchKernelGGL((sv_attn_group_kernel<T_, RM_, VC_>), grid, dim3(256), lds, st, a)
-#define SV_ATT_T(T_) do { if (vc == 1) SV_ATT(T_, 16, 1); else if (vc == 2) SV_ATT(T_, 16, 2); else if (vc == 4) SV_ATT(T_, 8, 4); else SV_ATT(T_, 4, 8); } while (0)
+#define SV_ATT_R(T_, VC_) do { if (rm == 2) SV_ATT(T_, 2, VC_); else if (rm == 4) SV_ATT(T_, 4, VC_); else if (rm == 8) SV_ATT(T_, 8, VC_); else SV_ATT(T_, 16, VC_); } while (0)
+#define SV_ATT_T(T_) do { if (vc == 1) SV_ATT_R(T_, 1); else if (vc == 2) SV_ATT_R(T_, 2); else if (vc == 4) { if (rm == 2) SV_ATT(T_, 2, 4); else if (rm == 4) SV_ATT(T_, 4, 4); else SV_ATT(T_, 8, 4); } \
+                          else { if (rm == 2) SV_ATT(T_, 2, 8); else SV_ATT(T_, 4, 8); } } while (0)
     if (f32) SV_ATT_T(float); else SV_ATT_T(uint16_t);
+    if (a.nsplit > 1) {
+        if (f32) hipLaunchKernelGGL(sv_attn_merge_kernel<float>, dim3(a.T, a.heads), dim3(64), 0, st, a);
+        else hipLaunchKernelGGL(sv_attn_merge_kernel<uint16_t>, dim3(a.T, a.heads), dim3(64), 0, st, a);
+    }
 #undef SV_ATT_T
+#undef SV_ATT_R
 #undef SV_ATT
 }
 
-void kr_sv_router(const void* h, bool f32, const float* gate, float* z, int T, int width, int E, int top, int groups, int keep, int renorm, int* ids, float* wts,
-                  hipStream_t st) {
+void kr_sv_router_select(const float* z, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st) {
     if (T <= 0) return;
-    const dim3 lgrid(T, (E + 15) / 16);
-    if (f32) hipLaunchKernelGGL(sv_router_logits_kernel<float>, lgrid, dim3(256), 0, st, (const float*)h, gate, width, E, z);
-    else hipLaunchKernelGGL(sv_router_logits_kernel<uint16_t>, lgrid, dim3(256), 0, st, (const uint16_t*)h, gate, width, E, z);
     const size_t lds = (size_t)(E + 2 * groups) * sizeof(float);
-    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, E, top, groups, keep, renorm, ids, wts);
+    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, parts, E, top, groups, keep, renorm, ids, wts);
 }
 
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st) {
     const int n = T * top;
     if (n <= 0) return;
+    if (n <= 1024 && E <= 4096) {
+        hipLaunchKernelGGL(sv_moe_sort_small_kernel, dim3(1), dim3(256), (size_t)2 * E * sizeof(int), st, ids, n, top, E, seg, src_row, row_group, pair_pos);
+        return;
+    }
     hipLaunchKernelGGL(sv_fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, st, counts, E, 0);
     hipLaunchKernelGGL(sv_moe_count_kernel, dim3((n + 255) / 256), dim3(256), 0, st, ids, n, counts);
     hipLaunchKernelGGL(sv_moe_scan_kernel, dim3(1), dim3(64), 0, st, counts, E, seg, cursor);
