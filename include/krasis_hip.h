@@ -412,6 +412,10 @@ int kr_serve_free_pages(kr_serve* s, int* n_out);
  * argmax_out: host i32 [n_want] or NULL.  KR_ERR_STATE when the pool has too few free pages (nothing is changed then). */
 int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* counts, const int* tokens, int n_want, const int* want_rows, float* logits_out,
                   int* argmax_out);
+/* Steps whose entries all bring one token (decode) replay a hipGraph captured at the second visit of their shape (batch, wanted rows, attention splits,
+ * scratch addresses); enable = 0 runs every step eagerly (same kernels, same results).  kr_serve_graph_replays counts the replayed steps. */
+int kr_serve_set_use_graph(kr_serve* s, int enable);
+long kr_serve_graph_replays(const kr_serve* s);
 /* the framework's sampler (kr_decode_sample's arithmetic) on wanted row `row` of the last step */
 int kr_serve_sample(kr_serve* s, int row, float temperature, int top_k, float top_p, uint64_t rng_seed, int* token_out);
 /* test aid: keep the residual stream after every layer of the next steps ([n_layers, T, width] f32), read it back */

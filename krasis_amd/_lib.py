@@ -29,7 +29,7 @@ SYMBOLS = [
     "kr_decode_weight_bytes",
     "kr_serve_create", "kr_serve_destroy", "kr_serve_set_tensor", "kr_serve_fill_synthetic", "kr_serve_finalize", "kr_serve_admit", "kr_serve_release",
     "kr_serve_slot_len", "kr_serve_free_pages", "kr_serve_step", "kr_serve_sample", "kr_serve_set_capture", "kr_serve_read_capture", "kr_serve_device_bytes",
-    "kr_serve_set_profiling", "kr_serve_get_profile",
+    "kr_serve_set_profiling", "kr_serve_get_profile", "kr_serve_set_use_graph", "kr_serve_graph_replays",
 ]
 TOKEN_CB = C.CFUNCTYPE(C.c_int, C.c_int, C.c_int, C.c_void_p)      # kr_token_cb(token, finish_reason, user) -> continue?
 
@@ -86,6 +86,8 @@ def _bind_serve(lib: C.CDLL) -> None:
     lib.kr_serve_device_bytes.argtypes = [vp]; lib.kr_serve_device_bytes.restype = C.c_size_t
     lib.kr_serve_set_profiling.argtypes = [vp, ci]
     lib.kr_serve_get_profile.argtypes = [vp, C.POINTER(C.c_double), ci]
+    lib.kr_serve_set_use_graph.argtypes = [vp, ci]
+    lib.kr_serve_graph_replays.argtypes = [vp]; lib.kr_serve_graph_replays.restype = C.c_long
 
 
 def load_serve_library(build: bool = False) -> C.CDLL:

@@ -19,8 +19,10 @@
 namespace {
 struct SvLayer {
     kr_serve_layer d{};
-    DevBuf norm_w, norm_b, qkv, o, sink, gu, down, router, egu, edown, sgu, sdown, kpool, vpool;
-    int rope_id = 0, n_qkv = 0;
+    // hw: every matrix that multiplies the normed input, row blocks [q | k | v | router | gate | up] (router: E rows, or hi + lo = 2E rows in a bf16
+    // store; gate | up: the dense feed-forward's or the shared expert's) -- one GEMM per layer produces them all
+    DevBuf norm_w, norm_b, hw, o, sink, down, egu, edown, sdown, kpool, vpool;
+    int rope_id = 0, n_qkv = 0, off_router = 0, n_router = 0, off_gu = 0, n_gu = 0, n_h = 0;
     std::vector<char> have;      // per role (expert roles: one flag per expert)
     int have_eg = 0, have_eu = 0, have_ed = 0;
     std::vector<char> eg, eu, ed;
@@ -52,6 +54,11 @@ struct kr_serve {
     // capture / profile
     bool capture = false; DevBuf cap; int cap_T = 0;
     bool prof = false; double prof_ms[8] = {0}; hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // decode-shaped steps repeat with the same launch sequence: captured once into a hipGraph, replayed afterwards
+    struct Graph { uint64_t key; hipGraphExec_t exec; };
+    std::vector<Graph> graphs;
+    std::vector<std::pair<uint64_t, int>> seen;      // keys met so far (a shape is captured at its second visit)
+    bool use_graph = true; long graph_replays = 0;
     // sampler scratch
     DevBuf s_keys, s_sorted, s_temp, s_probs, s_rng, s_tok, s_seen, s_row;
     size_t weight_bytes = 0;
@@ -152,6 +159,9 @@ int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_ser
         const kr_serve_layer& d = l.d;
         l.have.assign(KR_SV_N_ROLES, 0);
         l.n_qkv = d.heads * d.dim + (d.kv_from < 0 ? d.kv_heads * (d.dim + d.vdim) : 0);
+        l.n_router = d.mlp_kind == KR_SERVE_MLP_MOE ? d.experts * (s->f32 ? 1 : 2) : 0;
+        l.n_gu = d.mlp_kind == KR_SERVE_MLP_DENSE ? 2 * d.ff : (d.mlp_kind == KR_SERVE_MLP_MOE ? 2 * d.shared_ff : 0);
+        l.off_router = l.n_qkv; l.off_gu = l.off_router + l.n_router; l.n_h = l.off_gu + l.n_gu;
         if (d.mlp_kind == KR_SERVE_MLP_MOE) { l.eg.assign(d.experts, 0); l.eu.assign(d.experts, 0); l.ed.assign(d.experts, 0); }
         if (d.rot_dims > 0) {
             int id = -1;
@@ -183,6 +193,7 @@ void kr_serve_destroy(kr_serve* s) {
     if (s->ev0) (void)hipEventDestroy(s->ev0);
     if (s->ev1) (void)hipEventDestroy(s->ev1);
     if (s->h_meta) (void)hipHostFree(s->h_meta);
+    for (auto& g : s->graphs) (void)hipGraphExecDestroy(g.exec);
     delete s;
 }
 
@@ -211,31 +222,31 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     switch (role) {
     case KR_SV_NORM_W: SHAPE(1, W); rc = upload(s, l.norm_w, n, 0, host, src_dtype, n, true); break;
     case KR_SV_NORM_B: SHAPE(1, W); rc = upload(s, l.norm_b, n, 0, host, src_dtype, n, true); break;
-    case KR_SV_Q: SHAPE(nq, W); rc = upload(s, l.qkv, (size_t)l.n_qkv * W, 0, host, src_dtype, n, false); break;
+    case KR_SV_Q: SHAPE(nq, W); rc = upload(s, l.hw, (size_t)l.n_h * W, 0, host, src_dtype, n, false); break;
     case KR_SV_K: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its keys", layer);
-        SHAPE(nk, W); rc = upload(s, l.qkv, (size_t)l.n_qkv * W, (size_t)nq * W, host, src_dtype, n, false); break;
+        SHAPE(nk, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)nq * W, host, src_dtype, n, false); break;
     case KR_SV_V: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its values", layer);
-        SHAPE(nv, W); rc = upload(s, l.qkv, (size_t)l.n_qkv * W, (size_t)(nq + nk) * W, host, src_dtype, n, false); break;
+        SHAPE(nv, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)(nq + nk) * W, host, src_dtype, n, false); break;
     case KR_SV_O: SHAPE(W, d.heads * d.vdim); rc = upload(s, l.o, n, 0, host, src_dtype, n, false); break;
     case KR_SV_SINK: if (!d.has_sink) return kr_fail(KR_ERR_VALUE, "layer %d has no sink", layer);
         SHAPE(1, d.heads); rc = upload(s, l.sink, n, 0, host, src_dtype, n, true); break;
     case KR_SV_GATE: case KR_SV_UP:
         if (d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d has no dense feed-forward", layer);
-        SHAPE(d.ff, W); rc = upload(s, l.gu, (size_t)2 * d.ff * W, role == KR_SV_UP ? (size_t)d.ff * W : 0, host, src_dtype, n, false); break;
+        SHAPE(d.ff, W); rc = upload(s, l.hw, (size_t)l.n_h * W, ((size_t)l.off_gu + (role == KR_SV_UP ? d.ff : 0)) * W, host, src_dtype, n, false); break;
     case KR_SV_DOWN:
         if (d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d has no dense feed-forward", layer);
         SHAPE(W, d.ff); rc = upload(s, l.down, n, 0, host, src_dtype, n, false); break;
     case KR_SV_ROUTER: {
         if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no router", layer);
         SHAPE(d.experts, W);
-        if (s->f32) { rc = upload(s, l.router, n, 0, host, src_dtype, n, false); break; }
+        if (s->f32) { rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)l.off_router * W, host, src_dtype, n, false); break; }
         // bf16 store: gate = hi + lo, both bf16, rows [0, E) and [E, 2E) of one matrix
         std::vector<uint16_t> hl(2 * n);
         for (size_t k = 0; k < n; k++) {
             const float g = src_dtype == KR_SERVE_F32 ? ((const float*)host)[k] : bf16_to_f32_host(((const uint16_t*)host)[k]);
             hl[k] = f32_to_bf16_host(g); hl[n + k] = f32_to_bf16_host(g - bf16_to_f32_host(hl[k]));
         }
-        rc = upload(s, l.router, 2 * n, 0, hl.data(), KR_SERVE_BF16, 2 * n, false); break;
+        rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)l.off_router * W, hl.data(), KR_SERVE_BF16, 2 * n, false); break;
     }
     case KR_SV_EXPERT_GATE: case KR_SV_EXPERT_UP: case KR_SV_EXPERT_DOWN: {
         if (!moe) return kr_fail(KR_ERR_VALUE, "layer %d has no experts", layer);
@@ -251,7 +262,7 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     }
     case KR_SV_SHARED_GATE: case KR_SV_SHARED_UP:
         if (!moe || d.shared_ff < 1) return kr_fail(KR_ERR_VALUE, "layer %d has no shared expert", layer);
-        SHAPE(d.shared_ff, W); rc = upload(s, l.sgu, (size_t)2 * d.shared_ff * W, role == KR_SV_SHARED_UP ? (size_t)d.shared_ff * W : 0, host, src_dtype, n, false); break;
+        SHAPE(d.shared_ff, W); rc = upload(s, l.hw, (size_t)l.n_h * W, ((size_t)l.off_gu + (role == KR_SV_SHARED_UP ? d.shared_ff : 0)) * W, host, src_dtype, n, false); break;
     case KR_SV_SHARED_DOWN:
         if (!moe || d.shared_ff < 1) return kr_fail(KR_ERR_VALUE, "layer %d has no shared expert", layer);
         SHAPE(W, d.shared_ff); rc = upload(s, l.sdown, n, 0, host, src_dtype, n, false); break;
@@ -281,14 +292,13 @@ int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp) {
     s->have_embed = s->have_head = s->have_fw = s->have_fb = true;
     for (SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
-        bad |= vec(l.norm_w, W, true) | vec(l.norm_b, W, false) | mat(l.qkv, (size_t)l.n_qkv * W, W) | mat(l.o, (size_t)W * d.heads * d.vdim, d.heads * d.vdim);
+        bad |= vec(l.norm_w, W, true) | vec(l.norm_b, W, false) | mat(l.hw, (size_t)l.n_h * W, W) | mat(l.o, (size_t)W * d.heads * d.vdim, d.heads * d.vdim);
         if (d.has_sink) bad |= vec(l.sink, d.heads, false);
-        if (d.mlp_kind == KR_SERVE_MLP_DENSE) bad |= mat(l.gu, (size_t)2 * d.ff * W, W) | mat(l.down, (size_t)W * d.ff, d.ff);
+        if (d.mlp_kind == KR_SERVE_MLP_DENSE) bad |= mat(l.down, (size_t)W * d.ff, d.ff);
         if (d.mlp_kind == KR_SERVE_MLP_MOE) {
-            bad |= mat(l.router, (size_t)d.experts * W * (s->f32 ? 1 : 2), W);
-            if (!s->f32 && l.router.p) kr_sv_fill_uniform((uint16_t*)l.router.p + (size_t)d.experts * W, false, (size_t)d.experts * W, 0, 0.0f, s->st);   // lo rows: zero
+            if (!s->f32 && l.hw.p) kr_sv_fill_uniform((uint16_t*)l.hw.p + ((size_t)l.off_router + d.experts) * W, false, (size_t)d.experts * W, 0, 0.0f, s->st);   // the gate's lo rows: zero
             bad |= mat(l.egu, (size_t)d.experts * 2 * d.expert_ff * W, W) | mat(l.edown, (size_t)d.experts * W * d.expert_ff, d.expert_ff);
-            if (d.shared_ff > 0) bad |= mat(l.sgu, (size_t)2 * d.shared_ff * W, W) | mat(l.sdown, (size_t)W * d.shared_ff, d.shared_ff);
+            if (d.shared_ff > 0) bad |= mat(l.sdown, (size_t)W * d.shared_ff, d.shared_ff);
             std::fill(l.eg.begin(), l.eg.end(), 1); std::fill(l.eu.begin(), l.eu.end(), 1); std::fill(l.ed.begin(), l.ed.end(), 1);
         }
         std::fill(l.have.begin(), l.have.end(), 1);
@@ -414,7 +424,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0; int max_E = 1;
     for (const SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
-        max_qkv = std::max(max_qkv, (size_t)l.n_qkv); max_att = std::max(max_att, (size_t)d.heads * d.vdim);
+        max_qkv = std::max(max_qkv, (size_t)l.n_h); max_att = std::max(max_att, (size_t)d.heads * d.vdim);
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) { max_gu = std::max(max_gu, (size_t)2 * d.ff); max_y = std::max(max_y, (size_t)d.ff); }
         if (d.mlp_kind == KR_SERVE_MLP_MOE) {
             max_gu = std::max(max_gu, std::max((size_t)d.top * 2 * d.expert_ff, (size_t)2 * d.shared_ff));
@@ -430,6 +440,16 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         return kr_fail(KR_ERR_HIP, "step scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
     if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
+    std::vector<int> nsplit(c.n_layers, 1);
+    for (int li = 0; li < c.n_layers; li++) {
+        const kr_serve_layer& d = s->L[li].d;
+        nsplit[li] = kr_sv_attention_splits(T, d.heads, d.kv_heads, d.vdim, d.window > 0 ? std::min(max_pos + 1, d.window) : max_pos + 1);
+        if (nsplit[li] > 1 && (s->part_ml.ensure(Ts * d.heads * nsplit[li] * 8) || s->part_acc.ensure(Ts * d.heads * nsplit[li] * d.vdim * 4)))
+            return kr_fail(KR_ERR_HIP, "attention split scratch");
+    }
+    const bool want_amax = argmax_out != nullptr;
+    // every launch of the step, in order; no allocation, no host copy: the same body runs eagerly or under stream capture
+    auto enqueue = [&]() -> int {
     float* x = (float*)s->x.p;
     {
         Timer tm(s, 7);
@@ -440,24 +460,28 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         for (SvRope& r : s->ropes) kr_sv_rope_table(d_pos, (const double*)r.inv_freq.p, (float2*)r.cs.p, T, r.dims / 2, st);
     }
     int* mi = (int*)s->moe_i.p;
+    // down projection of a gated feed-forward: decode-sized problems form the activation inside the projection's launch, larger ones write it once
+    auto down_proj = [&](KrSvGemm g, const float* gu, int ld, int rows_m, int F, int kind, float limit, float alpha) {
+        if (kr_sv_gemm_small(g)) { g.act_gu = gu; g.act_ld = ld; g.act_kind = kind; g.act_limit = limit; g.act_alpha = alpha; g.A = nullptr; Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); return; }
+        { Timer tm(s, 5); kr_sv_act(gu, ld, s->y.p, s->f32, rows_m, F, kind, limit, alpha, st); }
+        g.A = s->y.p; g.lda = F;
+        { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+    };
+    { Timer tm(s, 0); kr_sv_norm(x, nullptr, (const float*)s->L[0].norm_w.p, (const float*)s->L[0].norm_b.p, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, st); }
     for (int li = 0; li < c.n_layers; li++) {
         SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
-        { Timer tm(s, 0); kr_sv_norm(x, nullptr, (const float*)l.norm_w.p, (const float*)l.norm_b.p, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, st); }
+        float* hz = (float*)s->qkv.p;                    // [T, n_h]: q | k | v | router logits | gate | up of this layer
         KrSvGemm g{};
-        g.A = s->h.p; g.lda = W; g.W = l.qkv.p; g.C = (float*)s->qkv.p; g.ldc = l.n_qkv; g.M = T; g.N = l.n_qkv; g.K = W;
+        g.A = s->h.p; g.lda = W; g.W = l.hw.p; g.C = hz; g.ldc = l.n_h; g.M = T; g.N = l.n_h; g.K = W;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         const SvLayer& kvl = d.kv_from >= 0 ? s->L[d.kv_from] : l;
         KrSvAttn a{};
-        a.qkv = (float*)s->qkv.p; a.ldq = l.n_qkv; a.heads = d.heads; a.kv_heads = d.kv_heads; a.dim = d.dim; a.vdim = d.vdim; a.rot_dims = d.rot_dims;
+        a.qkv = hz; a.ldq = l.n_h; a.heads = d.heads; a.kv_heads = d.kv_heads; a.dim = d.dim; a.vdim = d.vdim; a.rot_dims = d.rot_dims;
         a.rot_interleaved = d.rot_interleaved; a.unit_norm = d.qk_unit_norm; a.own_kv = d.kv_from < 0; a.eps = c.norm_eps; a.scale = d.scale; a.window = d.window;
         a.sink = d.has_sink ? (const float*)l.sink.p : nullptr; a.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
         a.kpool = kvl.kpool.p; a.vpool = kvl.vpool.p; a.page_table = d_tab; a.table_ld = s->n_pages; a.slot = d_slot; a.pos = d_pos; a.page_tokens = PT; a.T = T;
         a.out = s->att.p;
-        a.nsplit = kr_sv_attention_splits(T, d.heads, d.kv_heads, d.vdim, d.window > 0 ? std::min(max_pos + 1, d.window) : max_pos + 1);
-        if (a.nsplit > 1) {
-            if (s->part_ml.ensure(Ts * d.heads * a.nsplit * 8) || s->part_acc.ensure(Ts * d.heads * a.nsplit * d.vdim * 4)) return kr_fail(KR_ERR_HIP, "attention split scratch");
-            a.part_ml = (float*)s->part_ml.p; a.part_acc = (float*)s->part_acc.p;
-        }
+        a.nsplit = nsplit[li]; a.part_ml = (float*)s->part_ml.p; a.part_acc = (float*)s->part_acc.p;
         { Timer tm(s, 2); kr_sv_qk_prep(a, s->f32, st); }
         { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
         g = KrSvGemm{};
@@ -465,57 +489,94 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         const float *dense = nullptr, *shared = nullptr, *rows = nullptr; const int* pair_pos = nullptr;
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) {
-            g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.gu.p; g.C = (float*)s->gu.p; g.ldc = 2 * d.ff; g.M = T; g.N = 2 * d.ff; g.K = W;
-            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
-            { Timer tm(s, 5); kr_sv_act((const float*)s->gu.p, s->y.p, s->f32, T, d.ff, d.dense_act, 0.0f, 1.0f, st); }
-            g = KrSvGemm{}; g.A = s->y.p; g.lda = d.ff; g.W = l.down.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = d.ff;
-            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            g = KrSvGemm{}; g.W = l.down.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = d.ff;
+            down_proj(g, hz + l.off_gu, l.n_h, T, d.ff, d.dense_act, 0.0f, 1.0f);
             dense = (const float*)s->ffout.p;
         } else if (d.mlp_kind == KR_SERVE_MLP_MOE) {
             const int E = d.experts, top = d.top, F = d.expert_ff, P = T * top;
             int* counts_d = mi; int* seg = mi + E; int* cursor = seg + E + 1; int* src_row = cursor + E; int* row_group = src_row + P; int* pp = row_group + P;
             {
                 Timer tm(s, 4);
-                const int parts = s->f32 ? 1 : 2;
-                KrSvGemm rg{}; rg.A = s->h.p; rg.lda = W; rg.W = l.router.p; rg.C = (float*)s->rz.p; rg.ldc = parts * E; rg.M = T; rg.N = parts * E; rg.K = W;
-                kr_sv_gemm(rg, s->f32, st);
-                kr_sv_router_select((const float*)s->rz.p, parts, T, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
+                kr_sv_router_select(hz + l.off_router, l.n_h, s->f32 ? 1 : 2, T, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
                 kr_sv_moe_sort((const int*)s->ids.p, T, top, E, counts_d, seg, cursor, src_row, row_group, pp, st);
             }
             g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.egu.p; g.w_stride = (size_t)2 * F * W; g.C = (float*)s->gu.p; g.ldc = 2 * F; g.M = P; g.N = 2 * F; g.K = W;
             g.a_rows = src_row; g.seg = seg; g.row_group = row_group; g.n_groups = E;
             { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
-            { Timer tm(s, 5); kr_sv_act((const float*)s->gu.p, s->y.p, s->f32, P, F, d.expert_act, d.expert_limit, d.expert_alpha, st); }
-            g = KrSvGemm{}; g.A = s->y.p; g.lda = F; g.W = l.edown.p; g.w_stride = (size_t)W * F; g.C = (float*)s->rows.p; g.ldc = W; g.M = P; g.N = W; g.K = F;
+            g = KrSvGemm{}; g.W = l.edown.p; g.w_stride = (size_t)W * F; g.C = (float*)s->rows.p; g.ldc = W; g.M = P; g.N = W; g.K = F;
             g.seg = seg; g.row_group = row_group; g.n_groups = E;
-            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            down_proj(g, (const float*)s->gu.p, 2 * F, P, F, d.expert_act, d.expert_limit, d.expert_alpha);
             rows = (const float*)s->rows.p; pair_pos = pp;
             if (d.shared_ff > 0) {
                 const int SF = d.shared_ff;
-                g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.sgu.p; g.C = (float*)s->gu.p; g.ldc = 2 * SF; g.M = T; g.N = 2 * SF; g.K = W;
-                { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
-                { Timer tm(s, 5); kr_sv_act((const float*)s->gu.p, s->y.p, s->f32, T, SF, d.expert_act, d.shared_limit, d.expert_alpha, st); }
-                g = KrSvGemm{}; g.A = s->y.p; g.lda = SF; g.W = l.sdown.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = SF;
-                { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+                g = KrSvGemm{}; g.W = l.sdown.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = SF;
+                down_proj(g, hz + l.off_gu, l.n_h, T, SF, d.expert_act, d.shared_limit, d.expert_alpha);
                 shared = (const float*)s->ffout.p;
             }
         }
-        { Timer tm(s, 6); kr_sv_residual(x, (const float*)s->mix.p, dense, shared, rows, pair_pos, (const float*)s->wts.p, d.top, T, W, st); }
+        {   // x += mixer + feed-forward, and the next layer's normed input from the same launch
+            Timer tm(s, 6);
+            const SvLayer* nx = li + 1 < c.n_layers ? &s->L[li + 1] : nullptr;
+            kr_sv_residual_norm(x, (const float*)s->mix.p, dense, shared, rows, pair_pos, (const float*)s->wts.p, d.top, T, W, nx ? (const float*)nx->norm_w.p : nullptr,
+                                nx ? (const float*)nx->norm_b.p : nullptr, s->h.p, s->f32, c.norm_eps, c.norm_kind, st);
+        }
         if (s->capture) KR_HIP(hipMemcpyAsync((float*)s->cap.p + (size_t)li * Ts * W, x, Ts * W * 4, hipMemcpyDeviceToDevice, st));
     }
-    s->last_want = n_want;
     if (n_want > 0) {
         { Timer tm(s, 0); kr_sv_norm(x, d_want, (const float*)s->fnorm_w.p, (const float*)s->fnorm_b.p, s->hw.p, s->f32, n_want, W, c.norm_eps, c.norm_kind, st); }
         KrSvGemm g{}; g.A = s->hw.p; g.lda = W; g.W = s->head.p; g.C = (float*)s->logits.p; g.ldc = c.vocab; g.M = n_want; g.N = c.vocab; g.K = W;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
-        if (argmax_out) { Timer tm(s, 7); kr_sv_argmax((const float*)s->logits.p, n_want, c.vocab, (int*)s->amax.p, st); }
+        if (want_amax) { Timer tm(s, 7); kr_sv_argmax((const float*)s->logits.p, n_want, c.vocab, (int*)s->amax.p, st); }
+    }
+    return KR_OK;
+    };   // enqueue
+    bool decode_shaped = s->use_graph && !s->prof && !s->capture && T <= 64;
+    for (int e = 0; e < n_entries && decode_shaped; e++) decode_shaped = counts[e] == 1;
+    bool done = false;
+    if (decode_shaped) {
+        // the key: everything a launch argument depends on -- batch, wanted rows, the split of every layer, the scratch addresses
+        uint64_t key = 1469598103934665603ull;
+        auto mixin = [&](uint64_t v) { key = (key ^ v) * 1099511628211ull; };
+        mixin((uint64_t)T); mixin((uint64_t)n_want); mixin(want_amax);
+        for (int v : nsplit) mixin((uint64_t)v);
+        for (const DevBuf* b : {&s->meta, &s->x, &s->h, &s->qkv, &s->att, &s->mix, &s->gu, &s->y, &s->rows, &s->ffout, &s->ids, &s->wts, &s->rz, &s->moe_i, &s->hw, &s->logits,
+                                &s->amax, &s->part_ml, &s->part_acc}) mixin((uint64_t)(uintptr_t)b->p);
+        for (const SvRope& r : s->ropes) mixin((uint64_t)(uintptr_t)r.cs.p);
+        hipGraphExec_t exec = nullptr;
+        for (auto& g : s->graphs) if (g.key == key) exec = g.exec;
+        if (!exec) {
+            int visits = 0;
+            for (auto& q : s->seen) if (q.first == key) visits = ++q.second;
+            if (!visits) { if (s->seen.size() > 4096) s->seen.clear(); s->seen.emplace_back(key, 1); }
+            if (visits >= 2) {
+                if (s->graphs.size() >= 64) { for (auto& g : s->graphs) (void)hipGraphExecDestroy(g.exec); s->graphs.clear(); }
+                hipGraph_t graph = nullptr;
+                KR_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+                const int rc = enqueue();
+                const hipError_t ee = hipStreamEndCapture(st, &graph);
+                if (rc) { if (graph) (void)hipGraphDestroy(graph); return rc; }
+                if (ee != hipSuccess) return kr_fail(KR_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(ee));
+                const hipError_t ie = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+                (void)hipGraphDestroy(graph);
+                if (ie != hipSuccess) return kr_fail(KR_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(ie));
+                s->graphs.push_back({key, exec});
+            }
+        }
+        if (exec) { KR_HIP(hipGraphLaunch(exec, st)); s->graph_replays++; done = true; }
+    }
+    if (!done) { const int rc = enqueue(); if (rc) return rc; }
+    if (n_want > 0) {
         if (logits_out) KR_HIP(hipMemcpyAsync(logits_out, s->logits.p, (size_t)n_want * c.vocab * 4, hipMemcpyDeviceToHost, st));
         if (argmax_out) KR_HIP(hipMemcpyAsync(argmax_out, s->amax.p, (size_t)n_want * 4, hipMemcpyDeviceToHost, st));
     }
+    s->last_want = n_want;
     KR_HIP(hipStreamSynchronize(st));
     KR_HIP(hipGetLastError());
     return KR_OK;
 }
+
+int kr_serve_set_use_graph(kr_serve* s, int enable) { if (!s) return kr_fail(KR_ERR_VALUE, "null argument"); s->use_graph = enable != 0; return KR_OK; }
+long kr_serve_graph_replays(const kr_serve* s) { return s ? s->graph_replays : 0; }
 
 int kr_serve_sample(kr_serve* s, int row, float temperature, int top_k, float top_p, uint64_t rng_seed, int* token_out) {
     if (!s || !token_out) return kr_fail(KR_ERR_VALUE, "null argument");

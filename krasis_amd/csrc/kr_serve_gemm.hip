@@ -33,7 +33,16 @@ __device__ __forceinline__ bool gm_find_tile(const int* seg, int n_groups, int t
 }
 
 // ---------------------------------------------------------------------------------------------------------------- small M
-template <typename T, int MB>
+__device__ __forceinline__ float gm_act(float g, float u, int kind, float limit, float alpha) {
+    if (kind == KR_SV_ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+    if (kind == KR_SV_ACT_CLAMPED_SWIGLU) { g = fminf(g, limit); u = fminf(fmaxf(u, -limit), limit); return g / (1.0f + expf(-alpha * g)) * (u + 1.0f); }
+    return g / (1.0f + expf(-g)) * u;
+}
+template <typename T> __device__ __forceinline__ float gm_round(float v) { return v; }
+template <> __device__ __forceinline__ float gm_round<uint16_t>(float v) { return kr_bf16_to_f32(kr_f32_to_bf16(v)); }
+
+// ACT: the A operand is the gated activation of g.act_gu, formed as it is needed
+template <typename T, int MB, bool ACT>
 __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbase) {
     constexpr int VEC = 16 / sizeof(T);
     const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -43,16 +52,19 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
     if (g.row_group) { m0 = blockIdx.y; mcnt = 1; W += (size_t)g.row_group[m0] * g.w_stride; }
     else mcnt = min(MB, g.M - m0);
     const T* wr = W + (size_t)n * g.K;
-    const T* ar[MB];
+    const T* ar[MB]; const float* gr[MB];
 #pragma unroll
     for (int m = 0; m < MB; m++) {
         const int r = min(m0 + m, g.M - 1);
-        ar[m] = (const T*)g.A + (size_t)(g.a_rows ? g.a_rows[r] : r) * g.lda;
+        const int src = g.a_rows ? g.a_rows[r] : r;
+        ar[m] = ACT ? nullptr : (const T*)g.A + (size_t)src * g.lda;
+        gr[m] = ACT ? g.act_gu + (size_t)src * g.act_ld : nullptr;
     }
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; m++) acc[m] = 0.0f;
-    const bool vec = (g.K % VEC == 0) && (g.lda % VEC == 0) && (((uintptr_t)g.A | (uintptr_t)g.W) % 16 == 0) && (g.w_stride % VEC == 0);
+    const bool vec = ACT ? (g.K % VEC == 0) && (g.act_ld % 4 == 0) && (g.K % 4 == 0) && ((uintptr_t)g.act_gu % 16 == 0) && ((uintptr_t)g.W % 16 == 0) && (g.w_stride % VEC == 0)
+                         : (g.K % VEC == 0) && (g.lda % VEC == 0) && (((uintptr_t)g.A | (uintptr_t)g.W) % 16 == 0) && (g.w_stride % VEC == 0);
     if (vec) {
         for (int k = lane * VEC; k < g.K; k += 64 * VEC) {
             const gu4 wv = *reinterpret_cast<const gu4*>(wr + k);
@@ -67,6 +79,17 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
 #pragma unroll
             for (int m = 0; m < MB; m++) {
                 if (m < mcnt) {
+                    if constexpr (ACT) {
+#pragma unroll
+                        for (int q = 0; q < VEC / 4; q++) {
+                            const float4 gg = *reinterpret_cast<const float4*>(gr[m] + k + 4 * q), uu = *reinterpret_cast<const float4*>(gr[m] + g.K + k + 4 * q);
+                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.x, uu.x, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q], acc[m]);
+                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.y, uu.y, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q + 1], acc[m]);
+                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.z, uu.z, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q + 2], acc[m]);
+                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.w, uu.w, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q + 3], acc[m]);
+                        }
+                        continue;
+                    }
                     const gu4 av = *reinterpret_cast<const gu4*>(ar[m] + k);
                     if constexpr (sizeof(T) == 2) {
 #pragma unroll
@@ -85,7 +108,12 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
         for (int k = lane; k < g.K; k += 64) {
             const float w = gm_ld(wr + k);
 #pragma unroll
-            for (int m = 0; m < MB; m++) if (m < mcnt) acc[m] = __builtin_fmaf(gm_ld(ar[m] + k), w, acc[m]);
+            for (int m = 0; m < MB; m++) {
+                if (m < mcnt) {
+                    if constexpr (ACT) acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gr[m][k], gr[m][g.K + k], g.act_kind, g.act_limit, g.act_alpha)), w, acc[m]);
+                    else acc[m] = __builtin_fmaf(gm_ld(ar[m] + k), w, acc[m]);
+                }
+            }
         }
     }
 #pragma unroll
@@ -241,22 +269,26 @@ __global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
 }
 }  // namespace
 
+bool kr_sv_gemm_small(const KrSvGemm& g) {
+    // decode-sized problems: a pass over the weights per 8 rows; grouped problems take one row per workgroup row (each row has its own expert)
+    return g.seg ? (g.M <= 64 && g.row_group) : g.M <= 16;
+}
+
 void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st) {
     if (g.M <= 0 || g.N <= 0) return;
     const bool grouped = g.seg != nullptr;
-    // decode-sized problems: a pass over the weights per 8 rows; grouped problems take one row per workgroup row (each row has its own expert)
-    if ((!grouped && g.M <= 16) || (grouped && g.M <= 64 && g.row_group)) {
+    if (kr_sv_gemm_small(g)) {
+#define GM_V(T_, MB_, GRID_, ARG_, MBASE_) do { if (g.act_gu) hipLaunchKernelGGL((sv_gemv_kernel<T_, MB_, true>), GRID_, dim3(256), 0, st, ARG_, MBASE_); \
+                                                 else hipLaunchKernelGGL((sv_gemv_kernel<T_, MB_, false>), GRID_, dim3(256), 0, st, ARG_, MBASE_); } while (0)
         if (grouped) {
             const dim3 grid((g.N + 3) / 4, g.M);
-            if (f32) hipLaunchKernelGGL((sv_gemv_kernel<float, 1>), grid, dim3(256), 0, st, g, 0);
-            else hipLaunchKernelGGL((sv_gemv_kernel<uint16_t, 1>), grid, dim3(256), 0, st, g, 0);
+            if (f32) GM_V(float, 1, grid, g, 0); else GM_V(uint16_t, 1, grid, g, 0);
         } else {
             KrSvGemm p = g; p.row_group = nullptr;
-            for (int mb = 0; mb < g.M; mb += 8) {
-                if (f32) hipLaunchKernelGGL((sv_gemv_kernel<float, 8>), dim3((g.N + 3) / 4), dim3(256), 0, st, p, mb);
-                else hipLaunchKernelGGL((sv_gemv_kernel<uint16_t, 8>), dim3((g.N + 3) / 4), dim3(256), 0, st, p, mb);
-            }
+            const dim3 grid((g.N + 3) / 4);
+            for (int mb = 0; mb < g.M; mb += 8) { if (f32) GM_V(float, 8, grid, p, mb); else GM_V(uint16_t, 8, grid, p, mb); }
         }
+#undef GM_V
         return;
     }
     if (f32) {

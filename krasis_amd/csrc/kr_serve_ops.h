@@ -18,8 +18,12 @@ struct KrSvGemm {
     const int* seg;                  // grouped: [n_groups + 1] row offsets on the device (rows of group g are [seg[g], seg[g + 1])); null = one matrix
     const int* row_group;            // grouped: [M] group of every row (the small-M form reads it)
     int n_groups;
+    // small-M form only (kr_sv_gemm_small): A is not read but formed on the fly as the gated activation of act_gu [M, act_ld] f32 (gate at column k, up at
+    // column K + k), rounded to the storage type -- the down projection of a feed-forward without a launch and a buffer for the activation
+    const float* act_gu; int act_ld, act_kind; float act_limit, act_alpha;
 };
 void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st);
+bool kr_sv_gemm_small(const KrSvGemm& g);      // true: kr_sv_gemm takes the wave-per-column form for this problem (and honours act_gu)
 
 enum { KR_SV_NORM_LAYER = 0, KR_SV_NORM_RMS = 1 };
 enum { KR_SV_ACT_GELU_TANH = 0, KR_SV_ACT_CLAMPED_SWIGLU = 1, KR_SV_ACT_SILU = 2 };
@@ -50,18 +54,19 @@ int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_vis
 void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st);      // rotation, unit norm, cache append
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed softmax with an optional sink over the paged cache
 
-// group-limited top-k router on logits z [T, parts * E] f32 (the `parts` column blocks are added): softmax over all experts, the best `keep` of
+// group-limited top-k router on logits z (rows `ld` floats apart, `parts` column blocks of E that are added): softmax over all experts, the best `keep` of
 // `groups` groups (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum).
 // The logits come from kr_sv_gemm: an f32 store multiplies by the f32 gate; a bf16 store by the gate as two bf16 terms (hi + lo rows), which
 // carries 16 bits of the gate's mantissa through the matrix cores.
-void kr_sv_router_select(const float* z, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st);
+void kr_sv_router_select(const float* z, int ld, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st);
 // rows of every expert: seg[E + 1], src_row[T * top] (token of sorted row), row_group[T * top], pair_pos[T * top] (sorted row of (token, slot))
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st);
-// gu [M, 2F] f32 (gate | up) -> y [M, F] storage type
-void kr_sv_act(const float* gu, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st);
-// x[t] += mix[t] + (dense[t] + shared[t] + sum_s wts[t][s] * rows[pair_pos[t][s]]); null terms are skipped
-void kr_sv_residual(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
-                    int width, hipStream_t st);
+// gu rows `ld` floats apart (gate at [0, F), up at [F, 2F)) -> y [M, F] storage type
+void kr_sv_act(const float* gu, int ld, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st);
+// x[t] += mix[t] + (dense[t] + shared[t] + sum_s wts[t][s] * rows[pair_pos[t][s]]); null terms are skipped.  With norm_w the normed row of the NEW x
+// (the next layer's input) is written to h_out in the storage type by the same launch.
+void kr_sv_residual_norm(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
+                         int width, const float* norm_w, const float* norm_b, void* h_out, bool out_f32, float eps, int kind, hipStream_t st);
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st);
 // uniform values in [-amp, amp) from a counter hash of (seed, element); amp = 0 writes zeros
 void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, hipStream_t st);

@@ -213,7 +213,8 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
                 }
                 pc += PB;
             };
-            while (pc + 8 <= npiece) block(std::integral_constant<int, 8>{});
+            while (pc + 16 <= npiece) block(std::integral_constant<int, 16>{});
+            if (pc + 8 <= npiece) block(std::integral_constant<int, 8>{});
             if (pc + 4 <= npiece) block(std::integral_constant<int, 4>{});
             for (; pc < npiece; pc++) {
                 const sv_u4 kv = *reinterpret_cast<const sv_u4*>(k + pc * VEC);
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        constexpr int U = 16 / VC;                           // keys whose value rows are in flight together
+        constexpr int U = 32 / VC;                           // keys whose value rows are in flight together
         const int nk = min(64, p - j0 + 1);
         for (int jb = 0; jb < nk; jb += U) {                 // keys past nk inside the last group carry weight 0 and read the last key's row
             float vv[U][VC];
@@ -340,12 +341,12 @@ __global__ void __launch_bounds__(64) sv_attn_merge_kernel(const KrSvAttn a) {
 
 // selection: one wave per token; the scores of the E experts live in LDS
 // z holds the logits as `parts` column blocks of E that are added (a gate stored as two bf16 terms gives two)
-__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int parts, int E, int top, int groups, int keep, int renorm,
+__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int ld, int parts, int E, int top, int groups, int keep, int renorm,
                                                               int* __restrict__ ids, float* __restrict__ wts) {
     extern __shared__ float lds[];           // s[E] | gscore[groups] | allowed flags as floats [groups]
     float* s = lds; float* gs = lds + E; float* gok = gs + groups;
     const int t = blockIdx.x, lane = threadIdx.x;
-    for (int e = lane; e < E; e += 64) { float v = z[(size_t)t * parts * E + e]; for (int q = 1; q < parts; q++) v += z[((size_t)t * parts + q) * E + e]; s[e] = v; }
+    for (int e = lane; e < E; e += 64) { float v = z[(size_t)t * ld + e]; for (int q = 1; q < parts; q++) v += z[(size_t)t * ld + (size_t)q * E + e]; s[e] = v; }
     __syncthreads();
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
@@ -447,11 +448,11 @@ __global__ void __launch_bounds__(256) sv_moe_sort_small_kernel(const int* __res
 }
 
 template <typename T>
-__global__ void sv_act_kernel(const float* __restrict__ gu, T* __restrict__ y, int M, int F, int kind, float limit, float alpha) {
+__global__ void sv_act_kernel(const float* __restrict__ gu, int ld, T* __restrict__ y, int M, int F, int kind, float limit, float alpha) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)M * F) return;
     const size_t r = i / F; const int c = (int)(i - r * F);
-    float g = gu[r * 2 * F + c], u = gu[r * 2 * F + F + c], v;
+    float g = gu[r * ld + c], u = gu[r * ld + F + c], v;
     if (kind == KR_SV_ACT_GELU_TANH) {
         const float in = 0.7978845608028654f * (g + 0.044715f * g * g * g);
         v = 0.5f * g * (1.0f + tanhf(in)) * u;
@@ -464,21 +465,41 @@ __global__ void sv_act_kernel(const float* __restrict__ gu, T* __restrict__ y, i
     sv_st(y + i, v);
 }
 
-__global__ void sv_residual_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ dense, const float* __restrict__ shared,
-                                   const float* __restrict__ rows, const int* __restrict__ pair_pos, const float* __restrict__ wts, int top, int T, int width) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= (size_t)T * width) return;
-    const size_t t = i / width; const int c = (int)(i - t * width);
-    float ff = 0.0f; bool any = false;
-    if (rows) {
-        for (int s = 0; s < top; s++) ff = __builtin_fmaf(wts[t * top + s], rows[(size_t)pair_pos[t * top + s] * width + c], ff);
-        any = true;
+// one workgroup per token: the new residual row is formed in LDS, written back, and (with norm_w) normed from there for the next layer
+template <typename T, int KIND>
+__global__ void __launch_bounds__(256) sv_residual_norm_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ dense,
+                                                               const float* __restrict__ shared, const float* __restrict__ rows, const int* __restrict__ pair_pos,
+                                                               const float* __restrict__ wts, int top, int width, const float* __restrict__ norm_w,
+                                                               const float* __restrict__ norm_b, T* __restrict__ h_out, float eps) {
+    extern __shared__ float xr[];            // [width]
+    __shared__ float red[4];
+    const size_t t = blockIdx.x;
+    float s1 = 0.0f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        const size_t i = t * width + c;
+        float ff = 0.0f; bool any = false;
+        if (rows) {
+            for (int s = 0; s < top; s++) ff = __builtin_fmaf(wts[t * top + s], rows[(size_t)pair_pos[t * top + s] * width + c], ff);
+            any = true;
+        }
+        if (shared) { ff = any ? ff + shared[i] : shared[i]; any = true; }
+        if (dense) { ff = any ? ff + dense[i] : dense[i]; any = true; }
+        float d = mix ? mix[i] : 0.0f;
+        if (any) d = mix ? d + ff : ff;
+        const float v = x[i] + d;
+        x[i] = v; xr[c] = v; s1 += v;
     }
-    if (shared) { ff = any ? ff + shared[i] : shared[i]; any = true; }
-    if (dense) { ff = any ? ff + dense[i] : dense[i]; any = true; }
-    float d = mix ? mix[i] : 0.0f;
-    if (any) d = mix ? d + ff : ff;
-    x[i] += d;
+    if (!norm_w) return;
+    float mean = 0.0f;
+    if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }      // a thread re-reads its own columns
+    const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float v = (xr[c] - mean) * inv * norm_w[c];
+        if (norm_b) v += norm_b[c];
+        sv_st(h_out + t * width + c, v);
+    }
 }
 
 __global__ void __launch_bounds__(256) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
@@ -580,10 +601,10 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
 #undef SV_ATT
 }
 
-void kr_sv_router_select(const float* z, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st) {
+void kr_sv_router_select(const float* z, int ld, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st) {
     if (T <= 0) return;
     const size_t lds = (size_t)(E + 2 * groups) * sizeof(float);
-    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, parts, E, top, groups, keep, renorm, ids, wts);
+    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, ld, parts, E, top, groups, keep, renorm, ids, wts);
 }
 
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st) {
@@ -599,19 +620,22 @@ void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg
     hipLaunchKernelGGL(sv_moe_fill_kernel, dim3((n + 255) / 256), dim3(256), 0, st, ids, n, top, seg, cursor, src_row, row_group, pair_pos);
 }
 
-void kr_sv_act(const float* gu, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st) {
+void kr_sv_act(const float* gu, int ld, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st) {
     const size_t n = (size_t)M * F;
     if (n == 0) return;
     const dim3 grid((unsigned)((n + 255) / 256));
-    if (f32) hipLaunchKernelGGL(sv_act_kernel<float>, grid, dim3(256), 0, st, gu, (float*)y, M, F, kind, limit, alpha);
-    else hipLaunchKernelGGL(sv_act_kernel<uint16_t>, grid, dim3(256), 0, st, gu, (uint16_t*)y, M, F, kind, limit, alpha);
+    if (f32) hipLaunchKernelGGL(sv_act_kernel<float>, grid, dim3(256), 0, st, gu, ld, (float*)y, M, F, kind, limit, alpha);
+    else hipLaunchKernelGGL(sv_act_kernel<uint16_t>, grid, dim3(256), 0, st, gu, ld, (uint16_t*)y, M, F, kind, limit, alpha);
 }
 
-void kr_sv_residual(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
-                    int width, hipStream_t st) {
-    const size_t n = (size_t)T * width;
-    if (n == 0) return;
-    hipLaunchKernelGGL(sv_residual_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, x, mix, dense, shared, rows, pair_pos, wts, top, T, width);
+void kr_sv_residual_norm(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
+                         int width, const float* norm_w, const float* norm_b, void* h_out, bool out_f32, float eps, int kind, hipStream_t st) {
+    if (T <= 0) return;
+    const size_t lds = (size_t)width * sizeof(float);
+#define SV_RN(T_, K_) hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_>), dim3(T), dim3(256), lds, st, x, mix, dense, shared, rows, pair_pos, wts, top, width, norm_w, norm_b, (T_*)h_out, eps)
+    if (kind == KR_SV_NORM_LAYER) { if (out_f32) SV_RN(float, KR_SV_NORM_LAYER); else SV_RN(uint16_t, KR_SV_NORM_LAYER); }
+    else { if (out_f32) SV_RN(float, KR_SV_NORM_RMS); else SV_RN(uint16_t, KR_SV_NORM_RMS); }
+#undef SV_RN
 }
 
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st) {

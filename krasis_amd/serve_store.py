@@ -145,6 +145,12 @@ class ServeStore:
         check_serve(self._lib.kr_serve_read_capture(self._h, out.ctypes.data, out.size))
         return out
 
+    def set_use_graph(self, on: bool) -> None:
+        check_serve(self._lib.kr_serve_set_use_graph(self._h, int(on)))
+
+    def graph_replays(self) -> int:
+        return int(self._lib.kr_serve_graph_replays(self._h))
+
     def device_bytes(self) -> int:
         return int(self._lib.kr_serve_device_bytes(self._h))
 

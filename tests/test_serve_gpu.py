@@ -399,3 +399,30 @@ def test_store_refuses_what_it_cannot_run():
         st.finalize()                                         # tensors missing
     with pytest.raises(ValueError):
         st.set_tensor(0, "q", np.zeros((5, 32), np.float32))  # wrong shape
+
+
+def test_graph_replays_equal_eager_steps():
+    """decode steps replay a captured graph from their second visit on; every replay is compared with a store that runs eagerly, with eager steps of
+    other shapes (a prompt portion of a third request) and host synchronisation between the replays"""
+    cfg = cfg_wide(); W = O.random_weights(cfg, 41)
+    a, b = tokens(cfg, 150, 42), tokens(cfg, 150, 43)
+    c = tokens(cfg, 60, 44)
+    eng_g, eng_e = engine(cfg, W, "bfloat16"), engine(cfg, W, "bfloat16")
+    eng_e.store.set_use_graph(False)
+    for eng in (eng_g, eng_e):
+        eng.step([("a", a[:30], []), ("b", b[:7], [])])
+    for i in range(100):
+        entries = [("a", [a[30 + i]], [0]), ("b", [b[7 + i]], [0])]
+        lg, am = eng_g.step(entries)
+        le, ae = eng_e.step(entries)
+        assert np.array_equal(lg, le) and np.array_equal(am, ae), i
+        if i % 25 == 10:                                    # an eager step of another shape in between
+            part = c[(i // 25) * 15:(i // 25) * 15 + 15]
+            lg, _ = eng_g.step([("c", part, [14])]); le, _ = eng_e.step([("c", part, [14])])
+            assert np.array_equal(lg, le)
+    assert eng_g.store.graph_replays() >= 60 and eng_e.store.graph_replays() == 0
+    ref = O.forward(cfg, W, a[:130])[0]
+    lg, _ = eng_g.step([("a", [a[130]], [0])])
+    ref = O.forward(cfg, W, a[:131])[0]
+    e = np.sqrt(((lg[0] - ref[130]) ** 2).mean()) / np.sqrt((ref ** 2).mean())
+    assert e < 4e-2
