@@ -322,6 +322,169 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     }
 }
 
+// Prompt-sized steps: the same attention on the f32 matrix instruction (v_mfma_f32_16x16x4_f32: every product and sum stays f32).  A workgroup owns 16
+// query ROWS that share one key / value head -- the heads of its group for one token, or for 16 / R consecutive tokens of one request when the group has
+// fewer than 16 heads (a row carries its own position, so the causal and window masks are per row) -- and its four waves split the blocks of 64 keys.
+// Both products are formed TRANSPOSED so that nothing is shuffled between them:
+//   S^T[key][row] = K Q^T   (A = key rows, B = the rows' queries, held in registers for the whole launch)
+//   O^T[d][row]  += V^T P^T (A = value columns, B = the weights exactly where the first product left them: lane = row, register = key)
+// so a lane's accumulators all belong to ONE row and the online-softmax rescale is a per-lane scalar.  The reduction index of an MFMA is spread over the
+// four 16-lane groups; group q takes the CONTIGUOUS quarter q of a key row (dim / 4 elements, 16-byte loads) and the keys 4 q .. 4 q + 3 of a 16-key block.
+typedef float sv_f4 __attribute__((ext_vector_type(4)));
+template <typename T, int DQ, int DB>      // DQ = dim / 4 query elements per lane, DB = vdim / 16 value columns per lane
+__global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int VEC = 16 / sizeof(T);
+    const int G = a.kv_heads, R = a.heads / G, dim = DQ * 4, vdim = DB * 16;
+    const int Rb = R < 16 ? R : 16, TQ = 16 / Rb;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, row = lane & 15, qd = lane >> 4;
+    const int g = blockIdx.y, h_row = g * R + blockIdx.z * 16 + (row % Rb), t0 = blockIdx.x * TQ, tq_row = row / Rb;
+    float* ml = lds;                    // [4 waves][16 rows][2]
+    float* accs = lds + 4 * 16 * 2;     // [16 rows][vdim]
+    const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
+    for (int base = 0; base < TQ && t0 + base < a.T;) {
+        // the run of tokens [base, end) of this group that continue one request (same slot, consecutive positions)
+        const int sl = a.slot[t0 + base], p0 = a.pos[t0 + base];
+        int end = base + 1;
+        while (end < TQ && t0 + end < a.T && a.slot[t0 + end] == sl && a.pos[t0 + end] == p0 + (end - base)) end++;
+        const bool rv = tq_row >= base && tq_row < end;
+        const int p_row = rv ? p0 + (tq_row - base) : -1;
+        const int lo_row = a.window > 0 ? max(0, p_row - a.window + 1) : 0;
+        const int hi = p0 + (end - base - 1), lo = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
+        const int* table = a.page_table + (size_t)sl * a.table_ld;
+        float q[DQ];
+        {
+            const float* qp = a.qkv + (size_t)(t0 + (rv ? tq_row : base)) * a.ldq + (size_t)h_row * dim + qd * DQ;
+#pragma unroll
+            for (int i = 0; i < DQ; i++) q[i] = rv ? qp[i] * a.scale : 0.0f;
+        }
+        float m = -INFINITY, l = 0.0f;
+        sv_f4 acc[DB];
+#pragma unroll
+        for (int d = 0; d < DB; d++) acc[d] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        const int nch = (hi - lo) / 64 + 1;
+        for (int cb = wave; cb < nch; cb += 4) {
+            const int j0 = lo + 64 * cb;
+            // ---- S^T: four blocks of 16 keys
+            sv_f4 st[4];
+            int prow[4];
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++) {
+                const int key = min(j0 + kb * 16 + row, hi);         // keys past the last one are fetched again and masked
+                prow[kb] = table[key / a.page_tokens] * a.page_tokens + (key % a.page_tokens);
+            }
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++) {
+                const T* k = kp + ((size_t)prow[kb] * G + g) * dim + qd * DQ;
+                sv_u4 kv[DQ / VEC];
+#pragma unroll
+                for (int u = 0; u < DQ / VEC; u++) kv[u] = *reinterpret_cast<const sv_u4*>(k + u * VEC);
+                sv_f4 c = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int u = 0; u < DQ / VEC; u++) {
+                    float kf[VEC];
+                    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) { kf[2 * i] = __uint_as_float(kv[u][i] << 16); kf[2 * i + 1] = __uint_as_float(kv[u][i] & 0xFFFF0000u); }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) kf[i] = __uint_as_float(kv[u][i]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) c = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], q[u * VEC + i], c, 0, 0, 0);
+                }
+                st[kb] = c;
+            }
+            // ---- masks and the online softmax of this lane's row (its 16 keys here, the other 48 in the three lanes 16 apart)
+            float cm = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = j0 + kb * 16 + 4 * qd + i;
+                    const bool ok = rv && key <= p_row && key >= lo_row;
+                    st[kb][i] = ok ? st[kb][i] : -INFINITY;
+                    cm = fmaxf(cm, st[kb][i]);
+                }
+            cm = fmaxf(cm, __shfl_xor(cm, 16)); cm = fmaxf(cm, __shfl_xor(cm, 32));
+            const float mn = fmaxf(m, cm);
+            const float alpha = mn == -INFINITY ? 1.0f : expf(m - mn);       // a row that has seen no key yet keeps its zero state
+            float ps = 0.0f;
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) { const float pj = st[kb][i] == -INFINITY ? 0.0f : expf(st[kb][i] - mn); st[kb][i] = pj; ps += pj; }
+            ps += __shfl_xor(ps, 16); ps += __shfl_xor(ps, 32);
+            l = l * alpha + ps; m = mn;
+#pragma unroll
+            for (int d = 0; d < DB; d++) acc[d] *= alpha;
+            // ---- O^T += V^T P^T: key (kb, 4 qd + i) -> this lane reads its DB value columns of that key's row
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++) {
+                float vf[4][DB];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int pr = __shfl(prow[kb], 4 * qd + i);
+                    const T* vr = vp + ((size_t)pr * G + g) * vdim + row * DB;
+                    if constexpr ((DB * sizeof(T)) % 16 == 0) {
+#pragma unroll
+                        for (int u = 0; u < DB / VEC; u++) {
+                            const sv_u4 vv = *reinterpret_cast<const sv_u4*>(vr + u * VEC);
+                            if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                                for (int e = 0; e < 4; e++) { vf[i][u * VEC + 2 * e] = __uint_as_float(vv[e] << 16); vf[i][u * VEC + 2 * e + 1] = __uint_as_float(vv[e] & 0xFFFF0000u); }
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++) vf[i][u * VEC + e] = __uint_as_float(vv[e]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < DB; e++) vf[i][e] = sv_ld(vr + e);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int d = 0; d < DB; d++) acc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][d], st[kb][i], acc[d], 0, 0, 0);
+            }
+        }
+        // ---- the four waves' states -> one, in wave order; sink; output
+        __syncthreads();
+        if (qd == 0) { ml[(wave * 16 + row) * 2] = m; ml[(wave * 16 + row) * 2 + 1] = l; }
+        __syncthreads();
+        float M = -INFINITY;
+        for (int w = 0; w < 4; w++) M = fmaxf(M, ml[(w * 16 + row) * 2]);
+        if (a.sink) M = fmaxf(M, a.sink[h_row]);
+        const float f = m == -INFINITY ? 0.0f : expf(m - M);
+        for (int w = 0; w < 4; w++) {
+            if (wave == w) {
+#pragma unroll
+                for (int d = 0; d < DB; d++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int col = (4 * qd + i) * DB + d;
+                        accs[row * vdim + col] = (w == 0 ? 0.0f : accs[row * vdim + col]) + acc[d][i] * f;
+                    }
+            }
+            __syncthreads();
+        }
+        for (int i = tid; i < 16 * vdim; i += 256) {
+            const int r = i / vdim, tq = r / Rb;
+            if (tq < base || tq >= end) continue;
+            const int h = g * R + blockIdx.z * 16 + (r % Rb);
+            float Mr = -INFINITY;
+            for (int w = 0; w < 4; w++) Mr = fmaxf(Mr, ml[(w * 16 + r) * 2]);
+            if (a.sink) Mr = fmaxf(Mr, a.sink[h]);
+            float L = a.sink ? expf(a.sink[h] - Mr) : 0.0f;
+            for (int w = 0; w < 4; w++) { const float mw = ml[(w * 16 + r) * 2]; if (mw != -INFINITY) L += ml[(w * 16 + r) * 2 + 1] * expf(mw - Mr); }
+            sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), accs[i] / L);
+        }
+        __syncthreads();
+        base = end;
+    }
+}
+
 // the partial states of a split launch -> output: one wave per (token, head)
 template <typename T>
 __global__ void __launch_bounds__(64) sv_attn_merge_kernel(const KrSvAttn a) {
@@ -578,8 +741,39 @@ int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_vis
     return ns < 1 ? 1 : (int)ns;
 }
 
+// the matrix-instruction form takes prompt-sized steps whose head sizes fit its register tiling
+template <typename T>
+static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int R = a.heads / a.kv_heads;
+    if (a.T < 32 || a.nsplit != 1) return false;
+    if (!((R <= 16 && 16 % R == 0) || R % 16 == 0)) return false;
+    if (a.dim % (4 * VEC) != 0 || a.vdim % 16 != 0) return false;
+    const int Rb = R < 16 ? R : 16, TQ = 16 / Rb;
+    const dim3 grid((a.T + TQ - 1) / TQ, a.kv_heads, R <= 16 ? 1 : R / 16);
+    const size_t lds = (size_t)(4 * 16 * 2 + 16 * a.vdim) * sizeof(float);
+#define SV_MF(DQ_, DB_) do { hipLaunchKernelGGL((sv_attn_mfma_kernel<T, DQ_, DB_>), grid, dim3(256), lds, st, a); return true; } while (0)
+    const int dq = a.dim / 4, db = a.vdim / 16;
+    if (dq == 16 && db == 4) SV_MF(16, 4);
+    if (dq == 32 && db == 8) SV_MF(32, 8);
+    if (dq == 16 && db == 8) SV_MF(16, 8);
+    if (dq == 32 && db == 4) SV_MF(32, 4);
+    if (dq == 8 && db == 2) SV_MF(8, 2);
+    if (dq == 8 && db == 4) SV_MF(8, 4);
+    if (dq == 16 && db == 2) SV_MF(16, 2);
+    if (dq == 64 && db == 16) SV_MF(64, 16);
+    if (dq == 64 && db == 8) SV_MF(64, 8);
+    if (dq == 32 && db == 16) SV_MF(32, 16);
+    if (dq == 8 && db == 16) SV_MF(8, 16);
+    if (dq == 8 && db == 1) SV_MF(8, 1);
+    if (dq == 16 && db == 1) SV_MF(16, 1);
+#undef SV_MF
+    return false;
+}
+
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
+    if (f32 ? sv_attn_mfma_launch<float>(a, st) : sv_attn_mfma_launch<uint16_t>(a, st)) return;
     const int R = a.heads / a.kv_heads;
     const int vc = a.vdim <= 64 ? 1 : a.vdim <= 128 ? 2 : a.vdim <= 256 ? 4 : 8;
     const int rmax = vc <= 2 ? 16 : vc == 4 ? 8 : 4;       // RM * VC accumulators per lane stay within 32

@@ -244,8 +244,9 @@ def test_portions_of_several_sizes(sizes):
     assert rel(np.concatenate(rows), ref) < 2e-4
 
 
-def test_unequal_requests_in_one_batch_equal_each_alone():
-    cfg = cfg_varied(); W = O.random_weights(cfg, 27)
+@pytest.mark.parametrize("make", [cfg_varied, cfg_wide])
+def test_unequal_requests_in_one_batch_equal_each_alone(make):
+    cfg = make(); W = O.random_weights(cfg, 27)
     lens = {"a": 70, "b": 9, "c": 131, "d": 33}
     toks = {k: tokens(cfg, n, 30 + i) for i, (k, n) in enumerate(lens.items())}
     refs = {k: O.forward(cfg, W, t)[0] for k, t in toks.items()}
