@@ -401,7 +401,7 @@ def arch_compare(args):
             for b in range(B):
                 eng.step([(("d", b), toks(P), [])], logits=False)
             ent = lambda: [(("d", b), toks(1), [0]) for b in range(B)]
-            for _ in range(5):
+            for _ in range(20):
                 eng.step(ent(), logits=False)
             n = 50
             t0 = time.perf_counter()
