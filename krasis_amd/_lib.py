@@ -60,7 +60,7 @@ class ServeLayerC(C.Structure):
 
 _lib = None
 _serve_lib = None
-_SERVE_LIB = os.path.join(_HERE, "libkrasis_serve.so")
+_SERVE_LIB = os.environ.get("KRASIS_SERVE_LIB") or os.path.join(_HERE, "libkrasis_serve.so")   # KRASIS_SERVE_LIB: probe builds of the same library
 
 
 def lib_path() -> str:
@@ -97,7 +97,7 @@ def load_serve_library(build: bool = False) -> C.CDLL:
     global _serve_lib
     if _serve_lib is not None:
         return _serve_lib
-    if os.path.exists(_LIB):
+    if os.path.exists(_LIB) and not os.environ.get("KRASIS_SERVE_LIB"):
         full = load_library()
         if hasattr(full, "kr_serve_create"):
             _serve_lib = full

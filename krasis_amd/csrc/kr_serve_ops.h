@@ -48,6 +48,7 @@ struct KrSvAttn {
     void* out;                       // [T, heads * vdim] storage type
     int nsplit;                      // >= 1: workgroups that share a token's keys (few tokens: more of the chip per token); > 1 needs the two buffers below
     float* part_ml; float* part_acc; // [T][heads][nsplit][2] running (maximum, denominator), [T][heads][nsplit][vdim] unnormalised sums
+    int tq;                          // set by the launcher of the matrix-instruction form: tokens per workgroup
 };
 // how many ways to split: fills the chip when the step has few tokens; max_visible = most keys any token of the step sees in this layer
 int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_visible);

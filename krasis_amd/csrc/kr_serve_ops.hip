@@ -137,6 +137,12 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
 // the wave updates each head's running maximum / denominator (online softmax, f32) and the lanes then own value columns for p.v.  The four waves'
 // partial states are merged through LDS in wave order; the sink joins the denominator there, once.
 typedef uint32_t sv_u4 __attribute__((ext_vector_type(4)));
+#ifdef KR_SV_STAMPS      // probe build: shader-clock stamps of the first wave of the first workgroup (kr_sv_read_stamps)
+__device__ long long sv_stamps[16];
+#define SV_STAMP(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) sv_stamps[i] = __builtin_readcyclecounter(); } while (0)
+#else
+#define SV_STAMP(i) do { } while (0)
+#endif
 template <typename T, int RM, int VC>
 __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -154,8 +160,10 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     const float* q = a.qkv + (size_t)t * a.ldq + (size_t)h0 * dim;
     // heads past the group's last one are computed on zero queries and dropped: the loops below carry no per-head branches, so the loads of a block of
     // keys are all in flight before the first product needs them
+    SV_STAMP(0);
     for (int i = tid; i < RM * dim; i += 256) qs[i] = i < nr * dim ? q[i] * a.scale : 0.0f;
     __syncthreads();
+    SV_STAMP(1);
     const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
     float m[RM], l[RM], acc[RM][VC];
 #pragma unroll
@@ -186,6 +194,20 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         const int jc = min(j, p);                            // lanes past the last key score it again; their weight is set to 0
         const int prow = table[jc / a.page_tokens] * a.page_tokens + (jc % a.page_tokens);
         const T* k = kp + ((size_t)prow * G + g) * dim;
+        constexpr int U = 16 / VC;                           // keys whose value rows are requested together
+        const int nk = min(64, p - j0 + 1);
+        float va[U][VC], vb[U][VC];
+        auto fetch_v = [&](int jb, float (&vv)[U][VC]) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int pr = __builtin_amdgcn_readlane(prow, min(jb + u, 63));
+                const T* vr = vp + ((size_t)pr * G + g) * vdim;
+#pragma unroll
+                for (int c = 0; c < VC; c++) { const int d = lane + 64 * c; vv[u][c] = d < vdim ? sv_ld(vr + d) : 0.0f; }
+            }
+        };
+        SV_STAMP(2);
+        fetch_v(0, va);                                      // in flight behind the key rows, consumed after the softmax
         float s[RM];
 #pragma unroll
         for (int r = 0; r < RM; r++) s[r] = 0.0f;
@@ -232,6 +254,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
                 for (int r = 0; r < RM; r++) s[r] = __builtin_fmaf(qs[r * dim + d], kd, s[r]);
             }
         }
+        SV_STAMP(3);
 #pragma unroll
         for (int r = 0; r < RM; r++) {
             const float sr = live ? s[r] : -INFINITY;
@@ -248,27 +271,39 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        constexpr int U = 32 / VC;                           // keys whose value rows are in flight together
-        const int nk = min(64, p - j0 + 1);
-        for (int jb = 0; jb < nk; jb += U) {                 // keys past nk inside the last group carry weight 0 and read the last key's row
-            float vv[U][VC];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int pr = __builtin_amdgcn_readlane(prow, min(jb + u, 63));
-                const T* vr = vp + ((size_t)pr * G + g) * vdim;
-#pragma unroll
-                for (int c = 0; c < VC; c++) { const int d = lane + 64 * c; vv[u][c] = d < vdim ? sv_ld(vr + d) : 0.0f; }
-            }
+        SV_STAMP(4);
+        // groups of U keys: a group's products run while the next group's value rows are in flight (the first group's were requested before the scores);
+        // keys past nk inside the last group carry weight 0 and read the last key's row
+        auto products = [&](int jb, float (&vv)[U][VC]) {
 #pragma unroll
             for (int r = 0; r < RM; r++) {
+                if constexpr (U % 4 == 0) {      // four keys' weights per LDS read (jb is a multiple of U: the read is 16-byte aligned and stays inside the block)
 #pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const float w = pw[r * 64 + min(jb + u, 63)];
+                    for (int u4 = 0; u4 < U / 4; u4++) {
+                        const float4 w4 = *reinterpret_cast<const float4*>(&pw[r * 64 + jb + 4 * u4]);
 #pragma unroll
-                    for (int c = 0; c < VC; c++) acc[r][c] = __builtin_fmaf(w, vv[u][c], acc[r][c]);
+                        for (int c = 0; c < VC; c++) {
+                            acc[r][c] = __builtin_fmaf(w4.x, vv[4 * u4][c], acc[r][c]); acc[r][c] = __builtin_fmaf(w4.y, vv[4 * u4 + 1][c], acc[r][c]);
+                            acc[r][c] = __builtin_fmaf(w4.z, vv[4 * u4 + 2][c], acc[r][c]); acc[r][c] = __builtin_fmaf(w4.w, vv[4 * u4 + 3][c], acc[r][c]);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < U; u++) {
+                        const float w = pw[r * 64 + min(jb + u, 63)];
+#pragma unroll
+                        for (int c = 0; c < VC; c++) acc[r][c] = __builtin_fmaf(w, vv[u][c], acc[r][c]);
+                    }
                 }
             }
+        };
+        for (int jb = 0; jb < nk; jb += 2 * U) {
+            if (jb + U < nk) fetch_v(jb + U, vb);
+            products(jb, va);
+            if (jb + 2 * U < nk) fetch_v(jb + 2 * U, va);
+            if (jb + U < nk) products(jb + U, vb);
         }
+        SV_STAMP(5);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -278,6 +313,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         for (int r = 0; r < RM; r++) if (r < nr) { ml[(wave * RM + r) * 2] = m[r]; ml[(wave * RM + r) * 2 + 1] = l[r]; }
     }
     __syncthreads();
+    SV_STAMP(6);
     const bool last = a.nsplit == 1;                         // an unsplit launch finishes here: sink, normalisation, output; a split one leaves partial states
     float f[RM];
 #pragma unroll
@@ -320,6 +356,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
             if (i == r * vdim) { a.part_ml[slot * 2] = M; a.part_ml[slot * 2 + 1] = L; }
         }
     }
+    SV_STAMP(7);
 }
 
 // Prompt-sized steps: the same attention on the f32 matrix instruction (v_mfma_f32_16x16x4_f32: every product and sum stays f32).  A workgroup owns 16
@@ -336,11 +373,13 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int VEC = 16 / sizeof(T);
     const int G = a.kv_heads, R = a.heads / G, dim = DQ * 4, vdim = DB * 16;
-    const int Rb = R < 16 ? R : 16, TQ = 16 / Rb;
+    const int Rb = R < 16 ? R : 16, TQ = a.tq;             // tokens per workgroup: 16 / Rb for prompt portions, 1 for decode-shaped steps (rows past TQ * Rb idle)
+    const int sp = blockIdx.z % a.nsplit, hb = blockIdx.z / a.nsplit;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, row = lane & 15, qd = lane >> 4;
-    const int g = blockIdx.y, h_row = g * R + blockIdx.z * 16 + (row % Rb), t0 = blockIdx.x * TQ, tq_row = row / Rb;
+    const int g = blockIdx.y, h_row = g * R + hb * 16 + (row % Rb), t0 = blockIdx.x * TQ, tq_row = row / Rb;
     float* ml = lds;                    // [4 waves][16 rows][2]
-    float* accs = lds + 4 * 16 * 2;     // [16 rows][vdim]
+    float* mf = lds + 4 * 16 * 2;       // [16 rows][2]: the merged maximum and 1 / denominator (or the denominator itself in a split launch)
+    float* accs = mf + 16 * 2;          // [16 rows][vdim]
     const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
     for (int base = 0; base < TQ && t0 + base < a.T;) {
         // the run of tokens [base, end) of this group that continue one request (same slot, consecutive positions)
@@ -362,8 +401,8 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
         sv_f4 acc[DB];
 #pragma unroll
         for (int d = 0; d < DB; d++) acc[d] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
-        const int nch = (hi - lo) / 64 + 1;
-        for (int cb = wave; cb < nch; cb += 4) {
+        const int nch = (hi - lo) / 64 + 1, cps = (nch + a.nsplit - 1) / a.nsplit, c0 = sp * cps, c1 = min(nch, c0 + cps);
+        for (int cb = c0 + wave; cb < c1; cb += 4) {
             const int j0 = lo + 64 * cb;
             // ---- S^T: four blocks of 16 keys
             sv_f4 st[4];
@@ -449,14 +488,22 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
                     for (int d = 0; d < DB; d++) acc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][d], st[kb][i], acc[d], 0, 0, 0);
             }
         }
-        // ---- the four waves' states -> one, in wave order; sink; output
+        // ---- the four waves' states -> one, in wave order; an unsplit launch adds the sink and writes the output, a split one leaves (maximum, denominator, sums)
+        const bool last = a.nsplit == 1;
         __syncthreads();
         if (qd == 0) { ml[(wave * 16 + row) * 2] = m; ml[(wave * 16 + row) * 2 + 1] = l; }
         __syncthreads();
-        float M = -INFINITY;
-        for (int w = 0; w < 4; w++) M = fmaxf(M, ml[(w * 16 + row) * 2]);
-        if (a.sink) M = fmaxf(M, a.sink[h_row]);
-        const float f = m == -INFINITY ? 0.0f : expf(m - M);
+        if (tid < 16) {
+            const int h = g * R + hb * 16 + (tid % Rb);
+            float Mr = -INFINITY;
+            for (int w = 0; w < 4; w++) Mr = fmaxf(Mr, ml[(w * 16 + tid) * 2]);
+            if (last && a.sink) Mr = fmaxf(Mr, a.sink[h]);
+            float L = (last && a.sink) ? expf(a.sink[h] - Mr) : 0.0f;
+            for (int w = 0; w < 4; w++) { const float mw = ml[(w * 16 + tid) * 2]; if (mw != -INFINITY) L += ml[(w * 16 + tid) * 2 + 1] * expf(mw - Mr); }
+            mf[tid * 2] = Mr; mf[tid * 2 + 1] = last ? 1.0f / L : L;
+        }
+        __syncthreads();
+        const float f = m == -INFINITY ? 0.0f : expf(m - mf[row * 2]);
         for (int w = 0; w < 4; w++) {
             if (wave == w) {
 #pragma unroll
@@ -472,13 +519,13 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
         for (int i = tid; i < 16 * vdim; i += 256) {
             const int r = i / vdim, tq = r / Rb;
             if (tq < base || tq >= end) continue;
-            const int h = g * R + blockIdx.z * 16 + (r % Rb);
-            float Mr = -INFINITY;
-            for (int w = 0; w < 4; w++) Mr = fmaxf(Mr, ml[(w * 16 + r) * 2]);
-            if (a.sink) Mr = fmaxf(Mr, a.sink[h]);
-            float L = a.sink ? expf(a.sink[h] - Mr) : 0.0f;
-            for (int w = 0; w < 4; w++) { const float mw = ml[(w * 16 + r) * 2]; if (mw != -INFINITY) L += ml[(w * 16 + r) * 2 + 1] * expf(mw - Mr); }
-            sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), accs[i] / L);
+            const int h = g * R + hb * 16 + (r % Rb);
+            if (last) sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), accs[i] * mf[r * 2 + 1]);
+            else {
+                const size_t slot = ((size_t)(t0 + tq) * a.heads + h) * a.nsplit + sp;
+                a.part_acc[slot * vdim + (i - r * vdim)] = accs[i];
+                if (i == r * vdim) { a.part_ml[slot * 2] = mf[r * 2]; a.part_ml[slot * 2 + 1] = mf[r * 2 + 1]; }
+            }
         }
         __syncthreads();
         base = end;
@@ -746,13 +793,14 @@ template <typename T>
 static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
     constexpr int VEC = 16 / sizeof(T);
     const int R = a.heads / a.kv_heads;
-    if (a.T < 32 || a.nsplit != 1) return false;
     if (!((R <= 16 && 16 % R == 0) || R % 16 == 0)) return false;
     if (a.dim % (4 * VEC) != 0 || a.vdim % 16 != 0) return false;
-    const int Rb = R < 16 ? R : 16, TQ = 16 / Rb;
-    const dim3 grid((a.T + TQ - 1) / TQ, a.kv_heads, R <= 16 ? 1 : R / 16);
-    const size_t lds = (size_t)(4 * 16 * 2 + 16 * a.vdim) * sizeof(float);
-#define SV_MF(DQ_, DB_) do { hipLaunchKernelGGL((sv_attn_mfma_kernel<T, DQ_, DB_>), grid, dim3(256), lds, st, a); return true; } while (0)
+    const int Rb = R < 16 ? R : 16;
+    KrSvAttn b = a;
+    b.tq = a.nsplit > 1 ? 1 : 16 / Rb;      // a split launch is a decode-shaped step: its tokens belong to different requests
+    const dim3 grid((a.T + b.tq - 1) / b.tq, a.kv_heads, (R <= 16 ? 1 : R / 16) * a.nsplit);
+    const size_t lds = (size_t)(4 * 16 * 2 + 16 * 2 + 16 * a.vdim) * sizeof(float);
+#define SV_MF(DQ_, DB_) do { hipLaunchKernelGGL((sv_attn_mfma_kernel<T, DQ_, DB_>), grid, dim3(256), lds, st, b); return true; } while (0)
     const int dq = a.dim / 4, db = a.vdim / 16;
     if (dq == 16 && db == 4) SV_MF(16, 4);
     if (dq == 32 && db == 8) SV_MF(32, 8);
@@ -773,7 +821,13 @@ static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
 
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
-    if (f32 ? sv_attn_mfma_launch<float>(a, st) : sv_attn_mfma_launch<uint16_t>(a, st)) return;
+    if (f32 ? sv_attn_mfma_launch<float>(a, st) : sv_attn_mfma_launch<uint16_t>(a, st)) {
+        if (a.nsplit > 1) {
+            if (f32) hipLaunchKernelGGL(sv_attn_merge_kernel<float>, dim3(a.T, a.heads), dim3(64), 0, st, a);
+            else hipLaunchKernelGGL(sv_attn_merge_kernel<uint16_t>, dim3(a.T, a.heads), dim3(64), 0, st, a);
+        }
+        return;
+    }
     const int R = a.heads / a.kv_heads;
     const int vc = a.vdim <= 64 ? 1 : a.vdim <= 128 ? 2 : a.vdim <= 256 ? 4 : 8;
     const int rmax = vc <= 2 ? 16 : vc == 4 ? 8 : 4;       // RM * VC accumulators per lane stay within 32
@@ -836,3 +890,7 @@ void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t s
     if (R <= 0) return;
     hipLaunchKernelGGL(sv_argmax_kernel, dim3(R), dim3(256), 0, st, logits, vocab, out);
 }
+
+#ifdef KR_SV_STAMPS
+extern "C" int kr_sv_read_stamps(long long* out16) { return hipMemcpyFromSymbol(out16, HIP_SYMBOL(sv_stamps), sizeof(long long) * 16) != hipSuccess; }
+#endif
