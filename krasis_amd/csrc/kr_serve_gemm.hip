@@ -41,17 +41,20 @@ __device__ __forceinline__ float gm_act(float g, float u, int kind, float limit,
 template <typename T> __device__ __forceinline__ float gm_round(float v) { return v; }
 template <> __device__ __forceinline__ float gm_round<uint16_t>(float v) { return kr_bf16_to_f32(kr_f32_to_bf16(v)); }
 
-// ACT: the A operand is the gated activation of g.act_gu, formed as it is needed
-template <typename T, int MB, bool ACT>
+// ACT: the A operand is the gated activation of g.act_gu, formed as it is needed.  A wave owns CN consecutive output columns: their weight rows are
+// requested together (CN 16-byte reads in flight per k step), the input rows are read once for all of them.
+template <typename T, int MB, int CN, bool ACT>
 __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbase) {
     constexpr int VEC = 16 / sizeof(T);
-    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (n >= g.N) return;
+    const int lane = threadIdx.x & 63, n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * CN;
+    if (n0 >= g.N) return;
     int m0 = mbase, mcnt;
     const T* W = (const T*)g.W;
     if (g.row_group) { m0 = blockIdx.y; mcnt = 1; W += (size_t)g.row_group[m0] * g.w_stride; }
     else mcnt = min(MB, g.M - m0);
-    const T* wr = W + (size_t)n * g.K;
+    const T* wr[CN];
+#pragma unroll
+    for (int c = 0; c < CN; c++) wr[c] = W + (size_t)min(n0 + c, g.N - 1) * g.K;       // columns past N repeat the last one and are not stored
     const T* ar[MB]; const float* gr[MB];
 #pragma unroll
     for (int m = 0; m < MB; m++) {
@@ -60,69 +63,81 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
         ar[m] = ACT ? nullptr : (const T*)g.A + (size_t)src * g.lda;
         gr[m] = ACT ? g.act_gu + (size_t)src * g.act_ld : nullptr;
     }
-    float acc[MB];
+    float acc[MB][CN];
 #pragma unroll
-    for (int m = 0; m < MB; m++) acc[m] = 0.0f;
+    for (int m = 0; m < MB; m++)
+#pragma unroll
+        for (int c = 0; c < CN; c++) acc[m][c] = 0.0f;
     const bool vec = ACT ? (g.K % VEC == 0) && (g.act_ld % 4 == 0) && (g.K % 4 == 0) && ((uintptr_t)g.act_gu % 16 == 0) && ((uintptr_t)g.W % 16 == 0) && (g.w_stride % VEC == 0)
                          : (g.K % VEC == 0) && (g.lda % VEC == 0) && (((uintptr_t)g.A | (uintptr_t)g.W) % 16 == 0) && (g.w_stride % VEC == 0);
     if (vec) {
         for (int k = lane * VEC; k < g.K; k += 64 * VEC) {
-            const gu4 wv = *reinterpret_cast<const gu4*>(wr + k);
-            float wf[VEC];
-            if constexpr (sizeof(T) == 2) {
+            gu4 wv[CN];
 #pragma unroll
-                for (int i = 0; i < 4; i++) { wf[2 * i] = __uint_as_float(wv[i] << 16); wf[2 * i + 1] = __uint_as_float(wv[i] & 0xFFFF0000u); }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 4; i++) wf[i] = __uint_as_float(wv[i]);
-            }
+            for (int c = 0; c < CN; c++) wv[c] = *reinterpret_cast<const gu4*>(wr[c] + k);
 #pragma unroll
             for (int m = 0; m < MB; m++) {
                 if (m < mcnt) {
+                    float af[VEC];
                     if constexpr (ACT) {
 #pragma unroll
                         for (int q = 0; q < VEC / 4; q++) {
                             const float4 gg = *reinterpret_cast<const float4*>(gr[m] + k + 4 * q), uu = *reinterpret_cast<const float4*>(gr[m] + g.K + k + 4 * q);
-                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.x, uu.x, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q], acc[m]);
-                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.y, uu.y, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q + 1], acc[m]);
-                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.z, uu.z, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q + 2], acc[m]);
-                            acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gg.w, uu.w, g.act_kind, g.act_limit, g.act_alpha)), wf[4 * q + 3], acc[m]);
-                        }
-                        continue;
-                    }
-                    const gu4 av = *reinterpret_cast<const gu4*>(ar[m] + k);
-                    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            acc[m] = __builtin_fmaf(__uint_as_float(av[i] << 16), wf[2 * i], acc[m]);
-                            acc[m] = __builtin_fmaf(__uint_as_float(av[i] & 0xFFFF0000u), wf[2 * i + 1], acc[m]);
+                            af[4 * q] = gm_round<T>(gm_act(gg.x, uu.x, g.act_kind, g.act_limit, g.act_alpha)); af[4 * q + 1] = gm_round<T>(gm_act(gg.y, uu.y, g.act_kind, g.act_limit, g.act_alpha));
+                            af[4 * q + 2] = gm_round<T>(gm_act(gg.z, uu.z, g.act_kind, g.act_limit, g.act_alpha)); af[4 * q + 3] = gm_round<T>(gm_act(gg.w, uu.w, g.act_kind, g.act_limit, g.act_alpha));
                         }
                     } else {
+                        const gu4 av = *reinterpret_cast<const gu4*>(ar[m] + k);
+                        if constexpr (sizeof(T) == 2) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++) acc[m] = __builtin_fmaf(__uint_as_float(av[i]), wf[i], acc[m]);
+                            for (int i = 0; i < 4; i++) { af[2 * i] = __uint_as_float(av[i] << 16); af[2 * i + 1] = __uint_as_float(av[i] & 0xFFFF0000u); }
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) af[i] = __uint_as_float(av[i]);
+                        }
+                    }
+#pragma unroll
+                    for (int c = 0; c < CN; c++) {
+                        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                acc[m][c] = __builtin_fmaf(af[2 * i], __uint_as_float(wv[c][i] << 16), acc[m][c]);
+                                acc[m][c] = __builtin_fmaf(af[2 * i + 1], __uint_as_float(wv[c][i] & 0xFFFF0000u), acc[m][c]);
+                            }
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) acc[m][c] = __builtin_fmaf(af[i], __uint_as_float(wv[c][i]), acc[m][c]);
+                        }
                     }
                 }
             }
         }
     } else {
         for (int k = lane; k < g.K; k += 64) {
-            const float w = gm_ld(wr + k);
+            float w[CN];
+#pragma unroll
+            for (int c = 0; c < CN; c++) w[c] = gm_ld(wr[c] + k);
 #pragma unroll
             for (int m = 0; m < MB; m++) {
                 if (m < mcnt) {
-                    if constexpr (ACT) acc[m] = __builtin_fmaf(gm_round<T>(gm_act(gr[m][k], gr[m][g.K + k], g.act_kind, g.act_limit, g.act_alpha)), w, acc[m]);
-                    else acc[m] = __builtin_fmaf(gm_ld(ar[m] + k), w, acc[m]);
+                    float av;
+                    if constexpr (ACT) av = gm_round<T>(gm_act(gr[m][k], gr[m][g.K + k], g.act_kind, g.act_limit, g.act_alpha));
+                    else av = gm_ld(ar[m] + k);
+#pragma unroll
+                    for (int c = 0; c < CN; c++) acc[m][c] = __builtin_fmaf(av, w[c], acc[m][c]);
                 }
             }
         }
     }
 #pragma unroll
-    for (int m = 0; m < MB; m++) {
-        float v = acc[m];
+    for (int m = 0; m < MB; m++)
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-        if (lane == 0 && m < mcnt) g.C[(size_t)(m0 + m) * g.ldc + n] = v;
-    }
+        for (int c = 0; c < CN; c++) {
+            float v = acc[m][c];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+            if (lane == 0 && m < mcnt && n0 + c < g.N) g.C[(size_t)(m0 + m) * g.ldc + n0 + c] = v;
+        }
 }
 
 // ---------------------------------------------------------------------------------------------------------------- f32 tiles
@@ -278,15 +293,22 @@ void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st) {
     if (g.M <= 0 || g.N <= 0) return;
     const bool grouped = g.seg != nullptr;
     if (kr_sv_gemm_small(g)) {
-#define GM_V(T_, MB_, GRID_, ARG_, MBASE_) do { if (g.act_gu) hipLaunchKernelGGL((sv_gemv_kernel<T_, MB_, true>), GRID_, dim3(256), 0, st, ARG_, MBASE_); \
-                                                 else hipLaunchKernelGGL((sv_gemv_kernel<T_, MB_, false>), GRID_, dim3(256), 0, st, ARG_, MBASE_); } while (0)
+#define GM_V(T_, MB_, CN_, GRID_, ARG_, MBASE_) do { if (g.act_gu) hipLaunchKernelGGL((sv_gemv_kernel<T_, MB_, CN_, true>), GRID_, dim3(256), 0, st, ARG_, MBASE_); \
+                                                      else hipLaunchKernelGGL((sv_gemv_kernel<T_, MB_, CN_, false>), GRID_, dim3(256), 0, st, ARG_, MBASE_); } while (0)
+        // columns per wave: 4 while that still leaves a few waves for every SIMD of the chip, else 1
         if (grouped) {
-            const dim3 grid((g.N + 3) / 4, g.M);
-            if (f32) GM_V(float, 1, grid, g, 0); else GM_V(uint16_t, 1, grid, g, 0);
+            const bool wide = (long)g.N * g.M >= 8192;
+            const dim3 grid((g.N + (wide ? 15 : 3)) / (wide ? 16 : 4), g.M);
+            if (wide) { if (f32) GM_V(float, 1, 4, grid, g, 0); else GM_V(uint16_t, 1, 4, grid, g, 0); }
+            else { if (f32) GM_V(float, 1, 1, grid, g, 0); else GM_V(uint16_t, 1, 1, grid, g, 0); }
         } else {
             KrSvGemm p = g; p.row_group = nullptr;
-            const dim3 grid((g.N + 3) / 4);
-            for (int mb = 0; mb < g.M; mb += 8) { if (f32) GM_V(float, 8, grid, p, mb); else GM_V(uint16_t, 8, grid, p, mb); }
+            const bool wide = g.N >= 8192;
+            const dim3 grid((g.N + (wide ? 15 : 3)) / (wide ? 16 : 4));
+            for (int mb = 0; mb < g.M; mb += 8) {
+                if (wide) { if (f32) GM_V(float, 8, 4, grid, p, mb); else GM_V(uint16_t, 8, 4, grid, p, mb); }
+                else { if (f32) GM_V(float, 8, 1, grid, p, mb); else GM_V(uint16_t, 8, 1, grid, p, mb); }
+            }
         }
 #undef GM_V
         return;

@@ -683,13 +683,22 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(float* __restrict
                                                                const float* __restrict__ norm_b, T* __restrict__ h_out, float eps) {
     extern __shared__ float xr[];            // [width]
     __shared__ float red[4];
+    __shared__ int pp_s[64]; __shared__ float w_s[64];      // the token's expert rows and weights, read once (top <= 64; more fall back to global reads)
     const size_t t = blockIdx.x;
+    const bool staged = rows && top <= 64;
+    if (staged && threadIdx.x < top) { pp_s[threadIdx.x] = pair_pos[t * top + threadIdx.x]; w_s[threadIdx.x] = wts[t * top + threadIdx.x]; }
+    if (rows) __syncthreads();
     float s1 = 0.0f;
     for (int c = threadIdx.x; c < width; c += 256) {
         const size_t i = t * width + c;
         float ff = 0.0f; bool any = false;
         if (rows) {
-            for (int s = 0; s < top; s++) ff = __builtin_fmaf(wts[t * top + s], rows[(size_t)pair_pos[t * top + s] * width + c], ff);
+            if (staged) {
+#pragma unroll 4
+                for (int s = 0; s < top; s++) ff = __builtin_fmaf(w_s[s], rows[(size_t)pp_s[s] * width + c], ff);
+            } else {
+                for (int s = 0; s < top; s++) ff = __builtin_fmaf(wts[t * top + s], rows[(size_t)pair_pos[t * top + s] * width + c], ff);
+            }
             any = true;
         }
         if (shared) { ff = any ? ff + shared[i] : shared[i]; any = true; }
@@ -712,11 +721,12 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(float* __restrict
     }
 }
 
-__global__ void __launch_bounds__(256) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
-    __shared__ float bv[4]; __shared__ int bi[4];
+__global__ void __launch_bounds__(1024) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
+    __shared__ float bv[16]; __shared__ int bi[16];
     const float* row = logits + (size_t)blockIdx.x * vocab;
     float v = -INFINITY; int idx = 0x7fffffff;
-    for (int c = threadIdx.x; c < vocab; c += 256) { const float x = row[c]; if (x > v || (x == v && c < idx)) { v = x; idx = c; } }
+#pragma unroll 8
+    for (int c = threadIdx.x; c < vocab; c += 1024) { const float x = row[c]; if (x > v || (x == v && c < idx)) { v = x; idx = c; } }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(v, o); const int oi = __shfl_xor(idx, o);
@@ -725,7 +735,7 @@ __global__ void __launch_bounds__(256) sv_argmax_kernel(const float* __restrict_
     if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = v; bi[threadIdx.x >> 6] = idx; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; w++) if (bv[w] > v || (bv[w] == v && bi[w] < idx)) { v = bv[w]; idx = bi[w]; }
+        for (int w = 1; w < 16; w++) if (bv[w] > v || (bv[w] == v && bi[w] < idx)) { v = bv[w]; idx = bi[w]; }
         out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
     }
 }
@@ -888,7 +898,7 @@ void kr_sv_residual_norm(float* x, const float* mix, const float* dense, const f
 
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st) {
     if (R <= 0) return;
-    hipLaunchKernelGGL(sv_argmax_kernel, dim3(R), dim3(256), 0, st, logits, vocab, out);
+    hipLaunchKernelGGL(sv_argmax_kernel, dim3(R), dim3(1024), 0, st, logits, vocab, out);
 }
 
 #ifdef KR_SV_STAMPS
