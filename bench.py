@@ -385,6 +385,7 @@ def arch_compare(args):
             eng.store.set_profiling(profile)
             t0 = time.perf_counter(); eng.step([("p", toks(P), [P - 1])], logits=False); dt = time.perf_counter() - t0
             fam = eng.store.profile() if profile else None
+            eng.store.set_profiling(False)
             eng.finish("p")
             return dt, fam
         prompt_pass()

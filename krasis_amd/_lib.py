@@ -99,7 +99,7 @@ def load_serve_library(build: bool = False) -> C.CDLL:
         return _serve_lib
     if os.path.exists(_LIB) and not os.environ.get("KRASIS_SERVE_LIB"):
         full = load_library()
-        if hasattr(full, "kr_serve_create"):
+        if hasattr(full, "kr_serve_graph_replays"):          # a full library built before the serving store had all its entry points does not count
             _serve_lib = full
             return full
     if not os.path.exists(_SERVE_LIB):
@@ -243,7 +243,7 @@ def load_library() -> C.CDLL:
     lib.kr_decode_moe_route.argtypes = [vp, ci, vp, vp, vp, ci, ci, ci]
     lib.kr_decode_num_route_weights.argtypes = [vp]
     lib.kr_decode_weight_bytes.argtypes = [vp, ci]; lib.kr_decode_weight_bytes.restype = C.c_size_t
-    if hasattr(lib, "kr_serve_create"):
+    if hasattr(lib, "kr_serve_graph_replays"):
         _bind_serve(lib)
     _lib = lib
     return lib
