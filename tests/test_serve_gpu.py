@@ -95,6 +95,10 @@ def single_mechanism_model(mixer, mlp, width=64, vocab=50):
     ("experts_no_groups_no_shared", O.attn(2, 1, 8, 8, 0, 4, scale=0.3), O.moe(5, 2, 1, 1, 12, 0.8)),
     ("experts_groups_keep2_of_5", O.attn(2, 1, 8, 8, 0, 4, scale=0.3), O.moe(20, 3, 5, 2, 12, 1.7, 20, 0.6)),
     ("experts_top_equals_kept", O.attn(2, 1, 8, 8, 0, 4, scale=0.3), O.moe(8, 4, 2, 1, 12, 5.0, 8, 5.0)),
+    # shapes of the matrix-instruction attention: sixteen tokens of one head per workgroup; two batches of sixteen heads on one key head; wide values
+    ("one_head_per_key_head_window_9", O.attn(4, 4, 32, 16, 9, 8, scale=0.4), None),
+    ("thirty_two_heads_on_one_key_head", O.attn(32, 1, 32, 16, 11, 32, base=77.0, scale=0.4), None),
+    ("values_wider_than_keys", O.attn(8, 2, 32, 128, 0, 16, scale=0.3), None),
 ])
 def test_each_mechanism_alone(name, mixer, mlp):
     cfg = single_mechanism_model(mixer, mlp)
