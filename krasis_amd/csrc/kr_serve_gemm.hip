@@ -2,7 +2,7 @@
 // of a group contiguous, optional row gather for A).  Three forms:
 //   * small M (decode steps): one WAVE per output column, the K range over its lanes in 16-byte reads, up to 8 rows of A against one pass over
 //     the weight row -- bound by the weight stream;
-//   * bf16, larger M: workgroup tile 128 x 128 x 32 staged through LDS, four waves of 64 x 64 on v_mfma_f32_32x32x16_bf16, f32 accumulators, the next
+//   * bf16, larger M: workgroup tile 128 x 128 x 64 staged through LDS, four waves of 64 x 64 on v_mfma_f32_32x32x16_bf16, f32 accumulators, the next
 //     tile's global loads in flight during the MFMAs;
 //   * f32, larger M: 64 x 64 x 16 tile, 4 x 4 outputs per thread, plain fused multiply-adds (no reduced-precision matrix mode).
 // Every shape is accepted: edges are guarded, and rows whose byte length is not a multiple of 16 take element loads.
@@ -193,11 +193,13 @@ __global__ void __launch_bounds__(256) sv_gemm_f32_kernel(const KrSvGemm g) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------- bf16 tiles on the matrix cores
-#define GM_LD 40             // LDS row: 32 bf16 + 8 pad (80 bytes: 16-byte fragment reads of consecutive rows fall into distinct bank groups)
+#define GM_BK 64             // k depth of an LDS tile
+#define GM_KCH (GM_BK / 8)    // 16-byte chunks per tile row
+#define GM_LD (GM_BK + 8)    // LDS row: GM_BK bf16 + 8 pad (an odd number of 16-byte units: fragment reads of consecutive rows fall into distinct bank groups)
 template <int BM>            // 128 or 64 rows per workgroup; waves 2 x 2, each (BM / 2) x 64
 __global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
-    constexpr int BN = 128, BK = 32, MBW = BM / 64;      // 32-row blocks per wave
-    constexpr int ACH = BM * 4 / 256;                    // 16-byte chunks of the A tile per thread (rows x 4 chunks over 256 threads)
+    constexpr int BN = 128, BK = GM_BK, MBW = BM / 64;   // 32-row blocks per wave
+    constexpr int ACH = BM * GM_KCH / 256, BCH = BN * GM_KCH / 256;      // 16-byte chunks of the A / B tile per thread
     __shared__ __attribute__((aligned(16))) uint16_t As[BM * GM_LD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * GM_LD];
     int group = 0, m0 = blockIdx.y * BM, mend = g.M;
@@ -208,19 +210,19 @@ __global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
     const int wr = wave >> 1, wc = wave & 1;
     const bool vec = (g.K % 8 == 0) && (g.lda % 8 == 0) && (((uintptr_t)g.A | (uintptr_t)g.W) % 16 == 0) && (g.w_stride % 8 == 0);
-    const uint16_t* ap[ACH]; const uint16_t* bp[2];
-    int akc[ACH], bkc[2];
+    const uint16_t* ap[ACH]; const uint16_t* bp[BCH];
+    int akc[ACH], bkc[BCH];
 #pragma unroll
     for (int i = 0; i < ACH; i++) {
-        const int c = tid + i * 256, row = c >> 2;
-        akc[i] = (c & 3) * 8;
+        const int c = tid + i * 256, row = c / GM_KCH;
+        akc[i] = (c % GM_KCH) * 8;
         const int m = m0 + row;
         ap[i] = m < mend ? A + (size_t)(g.a_rows ? g.a_rows[m] : m) * g.lda : nullptr;
     }
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int c = tid + i * 256, row = c >> 2;
-        bkc[i] = (c & 3) * 8;
+    for (int i = 0; i < BCH; i++) {
+        const int c = tid + i * 256, row = c / GM_KCH;
+        bkc[i] = (c % GM_KCH) * 8;
         bp[i] = n0 + row < g.N ? W + (size_t)(n0 + row) * g.K : nullptr;
     }
     auto load16 = [&](const uint16_t* p, int k) -> gu4 {
@@ -238,26 +240,26 @@ __global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
         for (int b = 0; b < 2; b++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
-    gu4 ra[ACH], rb[2];
+    gu4 ra[ACH], rb[BCH];
 #pragma unroll
     for (int i = 0; i < ACH; i++) ra[i] = load16(ap[i], akc[i]);
 #pragma unroll
-    for (int i = 0; i < 2; i++) rb[i] = load16(bp[i], bkc[i]);
+    for (int i = 0; i < BCH; i++) rb[i] = load16(bp[i], bkc[i]);
     for (int k0 = 0; k0 < g.K; k0 += BK) {
         __syncthreads();                                 // the previous tile's fragment reads are done
 #pragma unroll
-        for (int i = 0; i < ACH; i++) { const int c = tid + i * 256; *reinterpret_cast<gu4*>(&As[(c >> 2) * GM_LD + akc[i]]) = ra[i]; }
+        for (int i = 0; i < ACH; i++) { const int c = tid + i * 256; *reinterpret_cast<gu4*>(&As[(c / GM_KCH) * GM_LD + akc[i]]) = ra[i]; }
 #pragma unroll
-        for (int i = 0; i < 2; i++) { const int c = tid + i * 256; *reinterpret_cast<gu4*>(&Bs[(c >> 2) * GM_LD + bkc[i]]) = rb[i]; }
+        for (int i = 0; i < BCH; i++) { const int c = tid + i * 256; *reinterpret_cast<gu4*>(&Bs[(c / GM_KCH) * GM_LD + bkc[i]]) = rb[i]; }
         __syncthreads();
         if (k0 + BK < g.K) {
 #pragma unroll
             for (int i = 0; i < ACH; i++) ra[i] = load16(ap[i], k0 + BK + akc[i]);
 #pragma unroll
-            for (int i = 0; i < 2; i++) rb[i] = load16(bp[i], k0 + BK + bkc[i]);
+            for (int i = 0; i < BCH; i++) rb[i] = load16(bp[i], k0 + BK + bkc[i]);
         }
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
+        for (int ks = 0; ks < BK / 16; ks++) {
             gb8 af[MBW], bf[2];
 #pragma unroll
             for (int a = 0; a < MBW; a++) af[a] = __builtin_bit_cast(gb8, *reinterpret_cast<const gu4*>(&As[(wr * (BM / 2) + a * 32 + r) * GM_LD + ks * 16 + h * 8]));
@@ -318,7 +320,8 @@ void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st) {
         hipLaunchKernelGGL(sv_gemm_f32_kernel, dim3((g.N + 63) / 64, tiles), dim3(256), 0, st, g);
         return;
     }
-    // grouped problems have few rows per expert: the 64-row tile wastes less of the matrix cores
+    // grouped problems have few rows per expert: the 64-row tile wastes less of the matrix cores.  (A 256-row tile -- wave tiles of 128 x 64, six fragment
+    // reads per eight MFMAs -- was measured and did not pay: two workgroups per compute unit instead of three.)
     const bool small = grouped ? (g.M / (g.n_groups > 0 ? g.n_groups : 1) < 96) : g.M <= 64;
     if (small) {
         const int tiles = grouped ? (g.M + 63) / 64 + g.n_groups : (g.M + 63) / 64;
