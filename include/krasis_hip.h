@@ -376,27 +376,70 @@ typedef struct {
     int dtype;                  /* KR_SERVE_BF16 | KR_SERVE_F32 */
     int norm_kind; float norm_eps;
     int max_slots, page_tokens, pool_tokens;   /* pool_tokens / page_tokens pages for all slots together */
+    /* how a layer is put together from its two sublayers (mixer, feed-forward):
+     *   KR_SERVE_BLOCK_PARALLEL    x += mult * (f(mixer(h)) + f(ff(h))), both on ONE input h
+     *   KR_SERVE_BLOCK_SEQUENTIAL  x += mult * f(mixer(h1)), then x += mult * f(ff(h2)) on the new x
+     * h = norm(x) with the layer's input norm (pre_norm) or x itself; f = the layer's output norm (post_norm, sequential blocks only) or nothing.
+     * norm_bias: the norms carry a bias tensor beside their weight.  All zero with residual_mult 1 and pre_norm 1 = one pre-normed parallel block. */
+    int block_kind, pre_norm, post_norm, norm_bias;
+    float residual_mult;
 } kr_serve_config;
 typedef struct {
-    /* mixer: attention with a parallel feed-forward on the same normed input (x += mixer(h) + ff(h)) */
+    /* mixer: attention over the paged cache; the feed-forward follows it or runs beside it (kr_serve_config.block_kind) */
     int heads, kv_heads, dim, vdim;
     int rot_dims, rot_interleaved;     /* rotary on the first rot_dims of a head; pairs (2i, 2i + 1) or (i, i + rot_dims / 2) */
     double rot_base, rot_factor;       /* f_i = base^(-2i / rot_dims) / factor */
-    int qk_unit_norm;                  /* q, k divided by their root mean square over dim after the rotation (eps = norm_eps) */
+    int qk_unit_norm;                  /* KR_SERVE_QKNORM_*: q, k divided by their root mean square over dim (eps = norm_eps) */
     float scale;
     int window;                        /* position i sees j with 0 <= i - j < window; 0 = all earlier positions */
-    int has_sink;                      /* softmax denominator + exp(sink[head]) */
+    int has_sink;                      /* KR_SERVE_SINK_*: softmax denominator + exp(sink[head]), or + 1 */
     int kv_from;                       /* -1, or the earlier layer whose cached keys / values this layer attends to (no k / v projections of its own) */
     int mlp_kind;
     int ff, dense_act;                 /* dense: down(act(gate h, up h)) */
     int experts, top, groups, keep, renorm;   /* router: softmax over all experts; best `keep` of `groups` groups; `top` experts; weights = scores */
     int expert_ff, expert_act; float expert_limit, expert_alpha;
     int shared_ff; float shared_limit;        /* 0 = no shared expert */
+    /* ---- mechanisms a design may switch on beside the ones above (all zero = off) */
+    int mixer_kind;                    /* KR_SERVE_MIX_ATTENTION | KR_SERVE_MIX_LATENT */
+    /* latent mixer: queries c_q = rms(W_dq h) * w -> q = W_uq c_q, per head [dim plain | rot_dims rotated]; W_dkv h = [kv_rank | rot_dims]: the first part,
+     * rms-normed with a weight, is the latent c, the second, rotated, one key part shared by all heads; per head k = [W_uk c | shared part], v = W_uv c.
+     * The cache holds c and the shared part only: a step folds W_uk into the queries and applies W_uv to the weighted sum of latents.  kv_heads is 1. */
+    int q_rank, kv_rank;
+    int rot_scaling;                   /* KR_SERVE_ROT_LINEAR (f / rot_factor) | KR_SERVE_ROT_BY_PARTS: pair i keeps f_i, is divided by rot_factor, or a blend: */
+    double rot_original, rot_fast, rot_slow;   /* pair(t) = rot_dims ln(rot_original / (2 pi t)) / (2 ln base); ramp from floor(pair(fast)) to ceil(pair(slow)); cos, sin * (0.1 ln factor + 1) */
+    int chunk;                         /* position i sees j <= i with floor(i / chunk) == floor(j / chunk); 0 = off (not together with window) */
+    int dist_bias; float dist_bias_exp;        /* score -= slope_h * (i - j), slope_h = 2^(-dist_bias_exp * (h + 1) / heads) */
+    int v_mix;                         /* KR_SERVE_VMIX_*: values blended with the values an earlier layer formed for the same token, before they are cached */
+    int router_bias;                   /* router logits + bias[expert] before the selection */
 } kr_serve_layer;
+#define KR_SERVE_BLOCK_PARALLEL 0
+#define KR_SERVE_BLOCK_SEQUENTIAL 1
+#define KR_SERVE_MIX_ATTENTION 0
+#define KR_SERVE_MIX_LATENT 1
+#define KR_SERVE_QKNORM_NONE 0
+#define KR_SERVE_QKNORM_AFTER_ROT 1    /* no weight, after the rotation */
+#define KR_SERVE_QKNORM_WEIGHTED 2     /* times a weight [dim] shared by the heads (tensors q_norm, k_norm), before the rotation */
+#define KR_SERVE_SINK_NONE 0
+#define KR_SERVE_SINK_TENSOR 1         /* learned score per head */
+#define KR_SERVE_SINK_ZERO 2           /* score 0: one added to the denominator */
+#define KR_SERVE_ROT_LINEAR 0
+#define KR_SERVE_ROT_BY_PARTS 1
+#define KR_SERVE_VMIX_NONE 0
+#define KR_SERVE_VMIX_FIRST 1          /* this layer's values are kept for the later mixing layers of the step */
+#define KR_SERVE_VMIX_BLEND 2          /* v <- (1 - l) v + l v_first, l = tensor vmix */
 /* tensor roles of kr_serve_set_tensor; layer = -1 for the first four */
 enum { KR_SV_EMBED = 0, KR_SV_FINAL_NORM_W, KR_SV_FINAL_NORM_B, KR_SV_HEAD, KR_SV_NORM_W, KR_SV_NORM_B, KR_SV_Q, KR_SV_K, KR_SV_V, KR_SV_O, KR_SV_SINK,
        KR_SV_GATE, KR_SV_UP, KR_SV_DOWN, KR_SV_ROUTER, KR_SV_EXPERT_GATE, KR_SV_EXPERT_UP, KR_SV_EXPERT_DOWN, KR_SV_SHARED_GATE, KR_SV_SHARED_UP,
-       KR_SV_SHARED_DOWN, KR_SV_N_ROLES };
+       KR_SV_SHARED_DOWN,
+       /* norm_w / norm_b above: input norm of the mixer (of both sublayers in a parallel block); NORM2: input norm of the feed-forward in a sequential
+        * block; POST1 / POST2: norms on the mixer's / the feed-forward's output */
+       KR_SV_NORM2_W, KR_SV_NORM2_B, KR_SV_POST1_W, KR_SV_POST1_B, KR_SV_POST2_W, KR_SV_POST2_B,
+       KR_SV_Q_NORM, KR_SV_K_NORM, KR_SV_VMIX, KR_SV_ROUTER_BIAS,
+       KR_SV_DQ, KR_SV_DQ_NORM, KR_SV_UQ, KR_SV_DKV, KR_SV_DKV_NORM, KR_SV_UK, KR_SV_UV,     /* latent mixer */
+       KR_SV_N_ROLES };
+/* layout version of kr_serve_config / kr_serve_layer: a caller built against another one must not use the library */
+#define KR_SERVE_ABI 2
+int kr_serve_abi(void);
 int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_serve_layer* layers, kr_serve** out);
 void kr_serve_destroy(kr_serve* s);
 /* host tensor [rows, cols] row-major ([out, in] for projections), src_dtype KR_SERVE_BF16 / KR_SERVE_F32; `index` = expert for the expert roles */

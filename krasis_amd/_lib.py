@@ -29,7 +29,7 @@ SYMBOLS = [
     "kr_decode_weight_bytes",
     "kr_serve_create", "kr_serve_destroy", "kr_serve_set_tensor", "kr_serve_fill_synthetic", "kr_serve_finalize", "kr_serve_admit", "kr_serve_release",
     "kr_serve_slot_len", "kr_serve_free_pages", "kr_serve_step", "kr_serve_sample", "kr_serve_set_capture", "kr_serve_read_capture", "kr_serve_device_bytes",
-    "kr_serve_set_profiling", "kr_serve_get_profile", "kr_serve_set_use_graph", "kr_serve_graph_replays",
+    "kr_serve_set_profiling", "kr_serve_get_profile", "kr_serve_set_use_graph", "kr_serve_graph_replays", "kr_serve_abi",
 ]
 TOKEN_CB = C.CFUNCTYPE(C.c_int, C.c_int, C.c_int, C.c_void_p)      # kr_token_cb(token, finish_reason, user) -> continue?
 
@@ -47,7 +47,8 @@ class ModelConfigC(C.Structure):
 
 class ServeConfigC(C.Structure):
     _fields_ = [("vocab", C.c_int), ("width", C.c_int), ("n_layers", C.c_int), ("dtype", C.c_int), ("norm_kind", C.c_int), ("norm_eps", C.c_float),
-                ("max_slots", C.c_int), ("page_tokens", C.c_int), ("pool_tokens", C.c_int)]
+                ("max_slots", C.c_int), ("page_tokens", C.c_int), ("pool_tokens", C.c_int),
+                ("block_kind", C.c_int), ("pre_norm", C.c_int), ("post_norm", C.c_int), ("norm_bias", C.c_int), ("residual_mult", C.c_float)]
 
 
 class ServeLayerC(C.Structure):
@@ -55,7 +56,12 @@ class ServeLayerC(C.Structure):
                 ("rot_base", C.c_double), ("rot_factor", C.c_double), ("qk_unit_norm", C.c_int), ("scale", C.c_float), ("window", C.c_int),
                 ("has_sink", C.c_int), ("kv_from", C.c_int), ("mlp_kind", C.c_int), ("ff", C.c_int), ("dense_act", C.c_int), ("experts", C.c_int),
                 ("top", C.c_int), ("groups", C.c_int), ("keep", C.c_int), ("renorm", C.c_int), ("expert_ff", C.c_int), ("expert_act", C.c_int),
-                ("expert_limit", C.c_float), ("expert_alpha", C.c_float), ("shared_ff", C.c_int), ("shared_limit", C.c_float)]
+                ("expert_limit", C.c_float), ("expert_alpha", C.c_float), ("shared_ff", C.c_int), ("shared_limit", C.c_float),
+                ("mixer_kind", C.c_int), ("q_rank", C.c_int), ("kv_rank", C.c_int), ("rot_scaling", C.c_int), ("rot_original", C.c_double), ("rot_fast", C.c_double),
+                ("rot_slow", C.c_double), ("chunk", C.c_int), ("dist_bias", C.c_int), ("dist_bias_exp", C.c_float), ("v_mix", C.c_int), ("router_bias", C.c_int)]
+
+
+SERVE_ABI = 2      # layout version of the two structures above (KR_SERVE_ABI in include/krasis_hip.h)
 
 
 _lib = None
@@ -88,6 +94,7 @@ def _bind_serve(lib: C.CDLL) -> None:
     lib.kr_serve_get_profile.argtypes = [vp, C.POINTER(C.c_double), ci]
     lib.kr_serve_set_use_graph.argtypes = [vp, ci]
     lib.kr_serve_graph_replays.argtypes = [vp]; lib.kr_serve_graph_replays.restype = C.c_long
+    lib.kr_serve_abi.argtypes = []
 
 
 def load_serve_library(build: bool = False) -> C.CDLL:
@@ -99,7 +106,7 @@ def load_serve_library(build: bool = False) -> C.CDLL:
         return _serve_lib
     if os.path.exists(_LIB) and not os.environ.get("KRASIS_SERVE_LIB"):
         full = load_library()
-        if hasattr(full, "kr_serve_graph_replays"):          # a full library built before the serving store had all its entry points does not count
+        if hasattr(full, "kr_serve_abi") and full.kr_serve_abi() == SERVE_ABI:      # a full library built before the serving store had this layout does not count
             _serve_lib = full
             return full
     if not os.path.exists(_SERVE_LIB):
@@ -112,6 +119,8 @@ def load_serve_library(build: bool = False) -> C.CDLL:
     if "torch" in sys.modules:
         import torch  # noqa: F401
     lib = C.CDLL(_SERVE_LIB)
+    if not hasattr(lib, "kr_serve_abi") or lib.kr_serve_abi() != SERVE_ABI:
+        raise KrasisHipError(f"{_SERVE_LIB} was built from other sources (structure layout {SERVE_ABI} expected): rebuild with `make -C krasis_amd/csrc serve`")
     _bind_serve(lib)
     _serve_lib = lib
     return lib
@@ -243,7 +252,7 @@ def load_library() -> C.CDLL:
     lib.kr_decode_moe_route.argtypes = [vp, ci, vp, vp, vp, ci, ci, ci]
     lib.kr_decode_num_route_weights.argtypes = [vp]
     lib.kr_decode_weight_bytes.argtypes = [vp, ci]; lib.kr_decode_weight_bytes.restype = C.c_size_t
-    if hasattr(lib, "kr_serve_graph_replays"):
+    if hasattr(lib, "kr_serve_abi"):
         _bind_serve(lib)
     _lib = lib
     return lib

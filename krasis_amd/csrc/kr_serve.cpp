@@ -21,13 +21,20 @@ struct SvLayer {
     kr_serve_layer d{};
     // hw: every matrix that multiplies the normed input, row blocks [q | k | v | router | gate | up] (router: E rows, or hi + lo = 2E rows in a bf16
     // store; gate | up: the dense feed-forward's or the shared expert's) -- one GEMM per layer produces them all
-    DevBuf norm_w, norm_b, hw, o, sink, down, egu, edown, sdown, kpool, vpool;
+    // A latent mixer's first row blocks are [dq | dkv] instead of [q | k | v]; its up-projections are matrices of their own: uq, and per head ukT
+    // [kv_rank, dim] (W_uk of the head transposed: it multiplies the QUERY) and uv [vdim, kv_rank].
+    DevBuf norm_w, norm_b, norm2_w, norm2_b, post1_w, post1_b, post2_w, post2_b, hw, o, sink, down, egu, edown, sdown, kpool, vpool;
+    DevBuf q_norm, k_norm, vmix, router_b, slopes, dq_norm, dkv_norm, uq, ukT, uv;
     int rope_id = 0, n_qkv = 0, off_router = 0, n_router = 0, off_gu = 0, n_gu = 0, n_h = 0;
+    bool latent() const { return d.mixer_kind == KR_SERVE_MIX_LATENT; }
+    int att_heads_kv() const { return latent() ? 1 : d.kv_heads; }
+    int att_dim() const { return latent() ? d.kv_rank + d.rot_dims : d.dim; }       // key row of the attention kernels
+    int att_vdim() const { return latent() ? d.kv_rank : d.vdim; }
     std::vector<char> have;      // per role (expert roles: one flag per expert)
     int have_eg = 0, have_eu = 0, have_ed = 0;
     std::vector<char> eg, eu, ed;
 };
-struct SvRope { int dims; double base, factor; DevBuf inv_freq; DevBuf cs; };
+struct SvRope { int dims, scaling; double base, factor, original, fast, slow; float mult; DevBuf inv_freq; DevBuf cs; };
 struct SvSlot { bool live = false; int len = 0; std::vector<int> pages; };
 }  // namespace
 
@@ -49,6 +56,8 @@ struct kr_serve {
     std::vector<int> h_table;
     // step scratch
     DevBuf meta, x, h, qkv, att, mix, gu, y, rows, ffout, ids, wts, rz, moe_i, hw, logits, amax, part_ml, part_acc;
+    DevBuf v_first;                                      // [T, kv_heads * vdim] f32: the values of the first value-mixing layer
+    DevBuf lq_c, lq_2, lq_n, lq_e, att2, head_i;         // latent mixer: query latent, W_uq output, plain query parts, folded queries, per-head values, head row tables
     void* h_meta = nullptr; size_t h_meta_bytes = 0;     // pinned staging of the per-step arrays
     int last_want = 0;
     // capture / profile
@@ -101,14 +110,32 @@ int check_layer(const kr_serve_config& c, const kr_serve_layer* all, int i) {
     const kr_serve_layer& d = all[i];
     if (d.heads < 1 || d.kv_heads < 1 || d.heads % d.kv_heads) return kr_fail(KR_ERR_VALUE, "layer %d: heads %d / kv_heads %d", i, d.heads, d.kv_heads);
     if (d.dim < 1 || d.vdim < 1 || d.vdim > 512 || d.dim > 512) return kr_fail(KR_ERR_VALUE, "layer %d: head sizes %d / %d (at most 512)", i, d.dim, d.vdim);
-    if (d.rot_dims < 0 || d.rot_dims > d.dim || (d.rot_dims & 1)) return kr_fail(KR_ERR_VALUE, "layer %d: rot_dims %d of %d", i, d.rot_dims, d.dim);
+    const bool lat = d.mixer_kind == KR_SERVE_MIX_LATENT;
+    if (d.mixer_kind != KR_SERVE_MIX_ATTENTION && !lat) return kr_fail(KR_ERR_VALUE, "layer %d: mixer kind %d", i, d.mixer_kind);
+    if (d.rot_dims < 0 || (!lat && d.rot_dims > d.dim) || (d.rot_dims & 1)) return kr_fail(KR_ERR_VALUE, "layer %d: rot_dims %d of %d", i, d.rot_dims, d.dim);
     if (d.rot_dims && (!(d.rot_base > 0.0) || !(d.rot_factor > 0.0))) return kr_fail(KR_ERR_VALUE, "layer %d: rotation base / factor", i);
-    if (d.window < 0) return kr_fail(KR_ERR_VALUE, "layer %d: window %d", i, d.window);
+    if (d.rot_scaling != KR_SERVE_ROT_LINEAR && d.rot_scaling != KR_SERVE_ROT_BY_PARTS) return kr_fail(KR_ERR_VALUE, "layer %d: rotation scaling %d", i, d.rot_scaling);
+    if (d.rot_dims && d.rot_scaling == KR_SERVE_ROT_BY_PARTS && (!(d.rot_original > 0.0) || !(d.rot_fast > 0.0) || !(d.rot_slow > 0.0) || !(d.rot_base > 1.0)))
+        return kr_fail(KR_ERR_VALUE, "layer %d: by-parts rotation scaling needs original, fast, slow > 0 and base > 1", i);
+    if (d.window < 0 || d.chunk < 0 || (d.window > 0 && d.chunk > 0)) return kr_fail(KR_ERR_VALUE, "layer %d: window %d / chunk %d", i, d.window, d.chunk);
+    if (d.qk_unit_norm < 0 || d.qk_unit_norm > KR_SERVE_QKNORM_WEIGHTED || d.has_sink < 0 || d.has_sink > KR_SERVE_SINK_ZERO || d.v_mix < 0 || d.v_mix > KR_SERVE_VMIX_BLEND)
+        return kr_fail(KR_ERR_VALUE, "layer %d: qk norm %d / sink %d / value mixing %d", i, d.qk_unit_norm, d.has_sink, d.v_mix);
+    if (lat) {
+        if (d.q_rank < 1 || d.kv_rank < 1 || d.kv_rank > 512 || d.kv_rank + d.rot_dims > 1024) return kr_fail(KR_ERR_VALUE, "layer %d: latent sizes %d / %d", i, d.q_rank, d.kv_rank);
+        if (d.kv_from >= 0 || d.v_mix || d.qk_unit_norm || d.kv_heads != 1) return kr_fail(KR_ERR_VALUE, "layer %d: a latent mixer has one latent per token, no borrowed cache, no value mixing, no q / k norm", i);
+    }
+    if (d.v_mix == KR_SERVE_VMIX_BLEND) {
+        int src = -1;
+        for (int j = 0; j < i; j++) if (all[j].v_mix == KR_SERVE_VMIX_FIRST) { src = j; break; }
+        if (src < 0) return kr_fail(KR_ERR_VALUE, "layer %d mixes values but no earlier layer keeps its own", i);
+        if (all[src].kv_heads * all[src].vdim != d.kv_heads * d.vdim) return kr_fail(KR_ERR_VALUE, "layer %d: values of layer %d have another size", i, src);
+    }
+    if (d.v_mix && d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d: value mixing needs values of its own", i);
     if (d.kv_from >= 0) {
         if (d.kv_from >= i) return kr_fail(KR_ERR_VALUE, "layer %d: kv_from %d is not an earlier layer", i, d.kv_from);
         const kr_serve_layer& o = all[d.kv_from];
         if (o.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d: kv_from %d has no cache of its own", i, d.kv_from);
-        if (o.kv_heads != d.kv_heads || o.dim != d.dim || o.vdim != d.vdim)
+        if (o.mixer_kind != d.mixer_kind || o.kv_heads != d.kv_heads || o.dim != d.dim || o.vdim != d.vdim)
             return kr_fail(KR_ERR_VALUE, "layer %d: key / value heads differ from layer %d", i, d.kv_from);
     }
     if (d.mlp_kind == KR_SERVE_MLP_DENSE && d.ff < 1) return kr_fail(KR_ERR_VALUE, "layer %d: ff %d", i, d.ff);
@@ -141,6 +168,8 @@ int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_ser
     if (cfg->dtype != KR_SERVE_BF16 && cfg->dtype != KR_SERVE_F32) return kr_fail(KR_ERR_VALUE, "dtype %d", cfg->dtype);
     if (cfg->norm_kind != KR_SERVE_NORM_LAYER && cfg->norm_kind != KR_SERVE_NORM_RMS) return kr_fail(KR_ERR_VALUE, "norm kind %d", cfg->norm_kind);
     if (cfg->max_slots < 1 || cfg->page_tokens < 1 || cfg->pool_tokens < cfg->page_tokens) return kr_fail(KR_ERR_VALUE, "slots / pages");
+    if (cfg->block_kind != KR_SERVE_BLOCK_PARALLEL && cfg->block_kind != KR_SERVE_BLOCK_SEQUENTIAL) return kr_fail(KR_ERR_VALUE, "block kind %d", cfg->block_kind);
+    if (cfg->post_norm && cfg->block_kind != KR_SERVE_BLOCK_SEQUENTIAL) return kr_fail(KR_ERR_VALUE, "norms on sublayer outputs need a sequential block");
     for (int i = 0; i < cfg->n_layers; i++) { const int rc = check_layer(*cfg, layers, i); if (rc) return rc; }
     int n_dev = 0;
     if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev <= device_ordinal) return kr_fail(KR_ERR_HIP, "no HIP device %d (the serving store has no CPU path)", device_ordinal);
@@ -158,27 +187,55 @@ int kr_serve_create(int device_ordinal, const kr_serve_config* cfg, const kr_ser
         SvLayer& l = s->L[i]; l.d = layers[i];
         const kr_serve_layer& d = l.d;
         l.have.assign(KR_SV_N_ROLES, 0);
-        l.n_qkv = d.heads * d.dim + (d.kv_from < 0 ? d.kv_heads * (d.dim + d.vdim) : 0);
+        l.n_qkv = l.latent() ? d.q_rank + d.kv_rank + d.rot_dims : d.heads * d.dim + (d.kv_from < 0 ? d.kv_heads * (d.dim + d.vdim) : 0);
         l.n_router = d.mlp_kind == KR_SERVE_MLP_MOE ? d.experts * (s->f32 ? 1 : 2) : 0;
         l.n_gu = d.mlp_kind == KR_SERVE_MLP_DENSE ? 2 * d.ff : (d.mlp_kind == KR_SERVE_MLP_MOE ? 2 * d.shared_ff : 0);
         l.off_router = l.n_qkv; l.off_gu = l.off_router + l.n_router; l.n_h = l.off_gu + l.n_gu;
         if (d.mlp_kind == KR_SERVE_MLP_MOE) { l.eg.assign(d.experts, 0); l.eu.assign(d.experts, 0); l.ed.assign(d.experts, 0); }
         if (d.rot_dims > 0) {
+            const bool parts = d.rot_scaling == KR_SERVE_ROT_BY_PARTS;
             int id = -1;
-            for (size_t r = 0; r < s->ropes.size(); r++) if (s->ropes[r].dims == d.rot_dims && s->ropes[r].base == d.rot_base && s->ropes[r].factor == d.rot_factor) id = (int)r;
+            for (size_t r = 0; r < s->ropes.size(); r++) {
+                const SvRope& q = s->ropes[r];
+                if (q.dims == d.rot_dims && q.base == d.rot_base && q.factor == d.rot_factor && q.scaling == d.rot_scaling &&
+                    (!parts || (q.original == d.rot_original && q.fast == d.rot_fast && q.slow == d.rot_slow))) id = (int)r;
+            }
             if (id < 0) {
-                s->ropes.emplace_back(); SvRope& r = s->ropes.back(); r.dims = d.rot_dims; r.base = d.rot_base; r.factor = d.rot_factor;
+                s->ropes.emplace_back(); SvRope& r = s->ropes.back(); r.dims = d.rot_dims; r.base = d.rot_base; r.factor = d.rot_factor; r.scaling = d.rot_scaling;
+                r.original = d.rot_original; r.fast = d.rot_fast; r.slow = d.rot_slow; r.mult = 1.0f;
                 std::vector<double> f(d.rot_dims / 2);
-                for (int k = 0; k < d.rot_dims / 2; k++) f[k] = std::pow(d.rot_base, -2.0 * k / d.rot_dims) / d.rot_factor;
+                if (!parts) {
+                    for (int k = 0; k < d.rot_dims / 2; k++) f[k] = std::pow(d.rot_base, -2.0 * k / d.rot_dims) / d.rot_factor;
+                } else {
+                    // pair index at which `turns` whole turns fit into `original` positions; pairs below lo keep their frequency, pairs above hi are divided
+                    // by the factor, a linear blend between; cos and sin are stretched by 0.1 ln(factor) + 1
+                    auto pair_of = [&](double turns) { return d.rot_dims * std::log(d.rot_original / (2.0 * M_PI * turns)) / (2.0 * std::log(d.rot_base)); };
+                    const double lo = std::max(std::floor(pair_of(d.rot_fast)), 0.0), hi = std::min(std::ceil(pair_of(d.rot_slow)), (double)(d.rot_dims - 1));
+                    for (int k = 0; k < d.rot_dims / 2; k++) {
+                        const double fk = std::pow(d.rot_base, -2.0 * k / d.rot_dims);
+                        const double ramp = std::min(std::max((k - lo) / std::max(hi - lo, 0.001), 0.0), 1.0);
+                        f[k] = fk / d.rot_factor * ramp + fk * (1.0 - ramp);
+                    }
+                    r.mult = (float)(0.1 * std::log(d.rot_factor) + 1.0);
+                }
                 if (r.inv_freq.ensure(f.size() * 8) || hipMemcpy(r.inv_freq.p, f.data(), f.size() * 8, hipMemcpyHostToDevice) != hipSuccess) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "rope table"); }
                 id = (int)s->ropes.size() - 1;
             }
             l.rope_id = id;
         }
+        if (d.dist_bias) {
+            std::vector<float> sl(d.heads);
+            for (int h = 0; h < d.heads; h++) sl[h] = (float)std::exp2(-(double)d.dist_bias_exp * (h + 1) / d.heads);
+            if (l.slopes.ensure(sl.size() * 4) || hipMemcpy(l.slopes.p, sl.data(), sl.size() * 4, hipMemcpyHostToDevice) != hipSuccess) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "slopes"); }
+        }
+        if (d.has_sink == KR_SERVE_SINK_ZERO) {
+            if (l.sink.ensure((size_t)d.heads * 4) || hipMemset(l.sink.p, 0, (size_t)d.heads * 4) != hipSuccess) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "sink"); }
+        }
         if (d.kv_from < 0) {
-            const size_t kb = (size_t)s->n_pages * cfg->page_tokens * d.kv_heads * d.dim * s->esz, vb = (size_t)s->n_pages * cfg->page_tokens * d.kv_heads * d.vdim * s->esz;
-            if (l.kpool.ensure(kb) || l.vpool.ensure(vb)) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "cache pool of %zu bytes", kb + vb); }
-            (void)hipMemset(l.kpool.p, 0, kb); (void)hipMemset(l.vpool.p, 0, vb);
+            const size_t rows = (size_t)s->n_pages * cfg->page_tokens;
+            const size_t kb = rows * l.att_heads_kv() * l.att_dim() * s->esz, vb = l.latent() ? 0 : rows * d.kv_heads * d.vdim * s->esz;     // a latent's values are its key rows
+            if (l.kpool.ensure(kb) || (vb && l.vpool.ensure(vb))) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "cache pool of %zu bytes", kb + vb); }
+            (void)hipMemset(l.kpool.p, 0, kb); if (vb) (void)hipMemset(l.vpool.p, 0, vb);
         }
     }
     if (s->page_table.ensure(s->h_table.size() * 4)) { kr_serve_destroy(s); return kr_fail(KR_ERR_HIP, "page table"); }
@@ -218,8 +275,41 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     const int nq = d.heads * d.dim, nk = d.kv_heads * d.dim, nv = d.kv_heads * d.vdim;
     if (role < 0 || role >= KR_SV_N_ROLES) return kr_fail(KR_ERR_VALUE, "role %d", role);
     const bool moe = d.mlp_kind == KR_SERVE_MLP_MOE;
+    const bool lat = l.latent();
+    if (lat && (role == KR_SV_Q || role == KR_SV_K || role == KR_SV_V)) return kr_fail(KR_ERR_VALUE, "layer %d has a latent mixer", layer);
+    if (!lat && role >= KR_SV_DQ && role <= KR_SV_UV) return kr_fail(KR_ERR_VALUE, "layer %d has no latent mixer", layer);
     int rc = KR_OK;
     switch (role) {
+    case KR_SV_NORM2_W: SHAPE(1, W); rc = upload(s, l.norm2_w, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_NORM2_B: SHAPE(1, W); rc = upload(s, l.norm2_b, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_POST1_W: SHAPE(1, W); rc = upload(s, l.post1_w, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_POST1_B: SHAPE(1, W); rc = upload(s, l.post1_b, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_POST2_W: SHAPE(1, W); rc = upload(s, l.post2_w, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_POST2_B: SHAPE(1, W); rc = upload(s, l.post2_b, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_Q_NORM: case KR_SV_K_NORM:
+        if (d.qk_unit_norm != KR_SERVE_QKNORM_WEIGHTED) return kr_fail(KR_ERR_VALUE, "layer %d has no weighted q / k norm", layer);
+        SHAPE(1, d.dim); rc = upload(s, role == KR_SV_Q_NORM ? l.q_norm : l.k_norm, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_VMIX: if (d.v_mix != KR_SERVE_VMIX_BLEND) return kr_fail(KR_ERR_VALUE, "layer %d blends no values", layer);
+        SHAPE(1, 1); rc = upload(s, l.vmix, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_ROUTER_BIAS: if (!moe || !d.router_bias) return kr_fail(KR_ERR_VALUE, "layer %d has no router bias", layer);
+        SHAPE(1, d.experts); rc = upload(s, l.router_b, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_DQ: SHAPE(d.q_rank, W); rc = upload(s, l.hw, (size_t)l.n_h * W, 0, host, src_dtype, n, false); break;
+    case KR_SV_DKV: SHAPE(d.kv_rank + d.rot_dims, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)d.q_rank * W, host, src_dtype, n, false); break;
+    case KR_SV_DQ_NORM: SHAPE(1, d.q_rank); rc = upload(s, l.dq_norm, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_DKV_NORM: SHAPE(1, d.kv_rank); rc = upload(s, l.dkv_norm, n, 0, host, src_dtype, n, true); break;
+    case KR_SV_UQ: SHAPE(d.heads * (d.dim + d.rot_dims), d.q_rank); rc = upload(s, l.uq, n, 0, host, src_dtype, n, false); break;
+    case KR_SV_UV: SHAPE(d.heads * d.vdim, d.kv_rank); rc = upload(s, l.uv, n, 0, host, src_dtype, n, false); break;
+    case KR_SV_UK: {      // [heads * dim, kv_rank] -> per head [kv_rank, dim]: the matrix that carries a head's plain query part into the latent space
+        SHAPE(d.heads * d.dim, d.kv_rank);
+        std::vector<float> tr(n);
+        for (int h = 0; h < d.heads; h++)
+            for (int e = 0; e < d.dim; e++)
+                for (int r = 0; r < d.kv_rank; r++) {
+                    const size_t src = ((size_t)h * d.dim + e) * d.kv_rank + r;
+                    tr[((size_t)h * d.kv_rank + r) * d.dim + e] = src_dtype == KR_SERVE_F32 ? ((const float*)host)[src] : bf16_to_f32_host(((const uint16_t*)host)[src]);
+                }
+        rc = upload(s, l.ukT, n, 0, tr.data(), KR_SERVE_F32, n, false); break;
+    }
     case KR_SV_NORM_W: SHAPE(1, W); rc = upload(s, l.norm_w, n, 0, host, src_dtype, n, true); break;
     case KR_SV_NORM_B: SHAPE(1, W); rc = upload(s, l.norm_b, n, 0, host, src_dtype, n, true); break;
     case KR_SV_Q: SHAPE(nq, W); rc = upload(s, l.hw, (size_t)l.n_h * W, 0, host, src_dtype, n, false); break;
@@ -228,7 +318,7 @@ int kr_serve_set_tensor(kr_serve* s, int layer, int role, int index, const void*
     case KR_SV_V: if (d.kv_from >= 0) return kr_fail(KR_ERR_VALUE, "layer %d borrows its values", layer);
         SHAPE(nv, W); rc = upload(s, l.hw, (size_t)l.n_h * W, (size_t)(nq + nk) * W, host, src_dtype, n, false); break;
     case KR_SV_O: SHAPE(W, d.heads * d.vdim); rc = upload(s, l.o, n, 0, host, src_dtype, n, false); break;
-    case KR_SV_SINK: if (!d.has_sink) return kr_fail(KR_ERR_VALUE, "layer %d has no sink", layer);
+    case KR_SV_SINK: if (d.has_sink != KR_SERVE_SINK_TENSOR) return kr_fail(KR_ERR_VALUE, "layer %d has no sink tensor", layer);
         SHAPE(1, d.heads); rc = upload(s, l.sink, n, 0, host, src_dtype, n, true); break;
     case KR_SV_GATE: case KR_SV_UP:
         if (d.mlp_kind != KR_SERVE_MLP_DENSE) return kr_fail(KR_ERR_VALUE, "layer %d has no dense feed-forward", layer);
@@ -288,15 +378,26 @@ int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp) {
         std::vector<float> h(n, one ? 1.0f : 0.0f);
         return hipMemcpy(b.p, h.data(), n * 4, hipMemcpyHostToDevice) != hipSuccess;
     };
-    int bad = mat(s->embed, (size_t)V * W, 1) | mat(s->head, (size_t)V * W, W) | vec(s->fnorm_w, W, true) | vec(s->fnorm_b, W, false);
+    const bool nb = s->c.norm_bias != 0;
+    int bad = mat(s->embed, (size_t)V * W, 1) | mat(s->head, (size_t)V * W, W) | vec(s->fnorm_w, W, true) | (nb ? vec(s->fnorm_b, W, false) : 0);
     s->have_embed = s->have_head = s->have_fw = s->have_fb = true;
     for (SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
-        bad |= vec(l.norm_w, W, true) | vec(l.norm_b, W, false) | mat(l.hw, (size_t)l.n_h * W, W) | mat(l.o, (size_t)W * d.heads * d.vdim, d.heads * d.vdim);
-        if (d.has_sink) bad |= vec(l.sink, d.heads, false);
+        bad |= mat(l.hw, (size_t)l.n_h * W, W) | mat(l.o, (size_t)W * d.heads * d.vdim, d.heads * d.vdim);
+        if (s->c.pre_norm) bad |= vec(l.norm_w, W, true) | (nb ? vec(l.norm_b, W, false) : 0);
+        if (s->c.pre_norm && s->c.block_kind == KR_SERVE_BLOCK_SEQUENTIAL) bad |= vec(l.norm2_w, W, true) | (nb ? vec(l.norm2_b, W, false) : 0);
+        if (s->c.post_norm) bad |= vec(l.post1_w, W, true) | vec(l.post2_w, W, true) | (nb ? vec(l.post1_b, W, false) | vec(l.post2_b, W, false) : 0);
+        if (d.has_sink == KR_SERVE_SINK_TENSOR) bad |= vec(l.sink, d.heads, false);
+        if (d.qk_unit_norm == KR_SERVE_QKNORM_WEIGHTED) bad |= vec(l.q_norm, d.dim, true) | vec(l.k_norm, d.dim, true);
+        if (d.v_mix == KR_SERVE_VMIX_BLEND) { bad |= vec(l.vmix, 1, true); const float half = 0.5f; bad |= hipMemcpy(l.vmix.p, &half, 4, hipMemcpyHostToDevice) != hipSuccess; }
+        if (l.latent()) {
+            bad |= vec(l.dq_norm, d.q_rank, true) | vec(l.dkv_norm, d.kv_rank, true) | mat(l.uq, (size_t)d.heads * (d.dim + d.rot_dims) * d.q_rank, d.q_rank) |
+                   mat(l.ukT, (size_t)d.heads * d.kv_rank * d.dim, d.kv_rank) | mat(l.uv, (size_t)d.heads * d.vdim * d.kv_rank, d.kv_rank);
+        }
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) bad |= mat(l.down, (size_t)W * d.ff, d.ff);
         if (d.mlp_kind == KR_SERVE_MLP_MOE) {
             if (!s->f32 && l.hw.p) kr_sv_fill_uniform((uint16_t*)l.hw.p + ((size_t)l.off_router + d.experts) * W, false, (size_t)d.experts * W, 0, 0.0f, s->st);   // the gate's lo rows: zero
+            if (d.router_bias) bad |= vec(l.router_b, d.experts, false);
             bad |= mat(l.egu, (size_t)d.experts * 2 * d.expert_ff * W, W) | mat(l.edown, (size_t)d.experts * W * d.expert_ff, d.expert_ff);
             if (d.shared_ff > 0) bad |= mat(l.sdown, (size_t)W * d.shared_ff, d.shared_ff);
             std::fill(l.eg.begin(), l.eg.end(), 1); std::fill(l.eu.begin(), l.eu.end(), 1); std::fill(l.ed.begin(), l.ed.end(), 1);
@@ -311,16 +412,28 @@ int kr_serve_fill_synthetic(kr_serve* s, uint64_t seed, float amp) {
 int kr_serve_finalize(kr_serve* s) {
     if (!s) return kr_fail(KR_ERR_VALUE, "null argument");
     if (!s->have_embed || !s->have_head || !s->have_fw) return kr_fail(KR_ERR_STATE, "embedding, head or final norm missing");
-    if (s->c.norm_kind == KR_SERVE_NORM_LAYER && !s->have_fb) return kr_fail(KR_ERR_STATE, "final norm bias missing");
+    if (s->c.norm_bias && !s->have_fb) return kr_fail(KR_ERR_STATE, "final norm bias missing");
+    const bool seq = s->c.block_kind == KR_SERVE_BLOCK_SEQUENTIAL, nb = s->c.norm_bias != 0;
     for (int i = 0; i < s->c.n_layers; i++) {
         SvLayer& l = s->L[i]; const kr_serve_layer& d = l.d;
-        std::vector<int> need = {KR_SV_NORM_W, KR_SV_Q, KR_SV_O};
-        if (s->c.norm_kind == KR_SERVE_NORM_LAYER) need.push_back(KR_SV_NORM_B);
-        if (d.kv_from < 0) { need.push_back(KR_SV_K); need.push_back(KR_SV_V); }
-        if (d.has_sink) need.push_back(KR_SV_SINK);
+        const bool has_ff = d.mlp_kind != KR_SERVE_MLP_NONE;
+        std::vector<int> need = {KR_SV_O};
+        if (s->c.pre_norm) { need.push_back(KR_SV_NORM_W); if (nb) need.push_back(KR_SV_NORM_B); }
+        if (s->c.pre_norm && seq && has_ff) { need.push_back(KR_SV_NORM2_W); if (nb) need.push_back(KR_SV_NORM2_B); }
+        if (s->c.post_norm) { need.push_back(KR_SV_POST1_W); if (nb) need.push_back(KR_SV_POST1_B); }
+        if (s->c.post_norm && has_ff) { need.push_back(KR_SV_POST2_W); if (nb) need.push_back(KR_SV_POST2_B); }
+        if (l.latent()) for (int r : {KR_SV_DQ, KR_SV_DQ_NORM, KR_SV_UQ, KR_SV_DKV, KR_SV_DKV_NORM, KR_SV_UK, KR_SV_UV}) need.push_back(r);
+        else {
+            need.push_back(KR_SV_Q);
+            if (d.kv_from < 0) { need.push_back(KR_SV_K); need.push_back(KR_SV_V); }
+        }
+        if (d.qk_unit_norm == KR_SERVE_QKNORM_WEIGHTED) { need.push_back(KR_SV_Q_NORM); if (d.kv_from < 0) need.push_back(KR_SV_K_NORM); }
+        if (d.v_mix == KR_SERVE_VMIX_BLEND) need.push_back(KR_SV_VMIX);
+        if (d.has_sink == KR_SERVE_SINK_TENSOR) need.push_back(KR_SV_SINK);
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) { need.push_back(KR_SV_GATE); need.push_back(KR_SV_UP); need.push_back(KR_SV_DOWN); }
         if (d.mlp_kind == KR_SERVE_MLP_MOE) {
             need.push_back(KR_SV_ROUTER);
+            if (d.router_bias) need.push_back(KR_SV_ROUTER_BIAS);
             if (d.shared_ff > 0) { need.push_back(KR_SV_SHARED_GATE); need.push_back(KR_SV_SHARED_UP); need.push_back(KR_SV_SHARED_DOWN); }
             for (int e = 0; e < d.experts; e++) if (!l.eg[e] || !l.eu[e] || !l.ed[e]) return kr_fail(KR_ERR_STATE, "layer %d: expert %d incomplete", i, e);
         }
@@ -329,6 +442,8 @@ int kr_serve_finalize(kr_serve* s) {
     s->finalized = true;
     return KR_OK;
 }
+
+int kr_serve_abi(void) { return KR_SERVE_ABI; }
 
 int kr_serve_admit(kr_serve* s, int* slot_out) {
     if (!s || !slot_out) return kr_fail(KR_ERR_VALUE, "null argument");
@@ -421,10 +536,17 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     const int* d_tok = (const int*)s->meta.p; const int* d_slot = d_tok + T; const int* d_pos = d_tok + 2 * T; const int* d_want = d_tok + 3 * T;
     const int* d_tab = d_tok + n_meta;
     // ---- scratch sized for this step
-    size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0; int max_E = 1;
+    const bool seq = c.block_kind == KR_SERVE_BLOCK_SEQUENTIAL;
+    size_t max_qkv = 0, max_att = 0, max_gu = 0, max_y = 0, max_rows = 0, max_pairs = 0, max_vf = 0; int max_E = 1;
+    size_t lq_c = 0, lq_2 = 0, lq_n = 0, lq_e = 0, att2 = 0, head_i = 0;
     for (const SvLayer& l : s->L) {
         const kr_serve_layer& d = l.d;
-        max_qkv = std::max(max_qkv, (size_t)l.n_h); max_att = std::max(max_att, (size_t)d.heads * d.vdim);
+        max_qkv = std::max(max_qkv, (size_t)l.n_h); max_att = std::max(max_att, (size_t)d.heads * l.att_vdim());
+        if (d.v_mix) max_vf = std::max(max_vf, (size_t)d.kv_heads * d.vdim);
+        if (l.latent()) {
+            lq_c = std::max(lq_c, (size_t)d.q_rank); lq_2 = std::max(lq_2, (size_t)d.heads * (d.dim + d.rot_dims)); lq_n = std::max(lq_n, (size_t)d.heads * d.dim);
+            lq_e = std::max(lq_e, (size_t)d.heads * l.att_dim()); att2 = std::max(att2, (size_t)d.heads * d.vdim); head_i = std::max(head_i, (size_t)d.heads);
+        }
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) { max_gu = std::max(max_gu, (size_t)2 * d.ff); max_y = std::max(max_y, (size_t)d.ff); }
         if (d.mlp_kind == KR_SERVE_MLP_MOE) {
             max_gu = std::max(max_gu, std::max((size_t)d.top * 2 * d.expert_ff, (size_t)2 * d.shared_ff));
@@ -438,13 +560,18 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         s->ids.ensure(Ts * max_pairs * 4 + 16) || s->rz.ensure(Ts * (size_t)max_E * 8 + 16) || s->wts.ensure(Ts * max_pairs * 4 + 16) || s->moe_i.ensure((Ts * max_pairs * 3 + 3 * (size_t)max_E + 8) * 4) ||
         s->hw.ensure((size_t)std::max(n_want, 1) * W * s->esz) || s->logits.ensure((size_t)std::max(n_want, 1) * c.vocab * 4) || s->amax.ensure((size_t)std::max(n_want, 1) * 4))
         return kr_fail(KR_ERR_HIP, "step scratch for %d tokens", T);
+    if ((max_vf && s->v_first.ensure(Ts * max_vf * 4)) ||
+        (head_i && (s->lq_c.ensure(Ts * lq_c * s->esz) || s->lq_2.ensure(Ts * lq_2 * 4) || s->lq_n.ensure(Ts * lq_n * s->esz) || s->lq_e.ensure(Ts * lq_e * 4) ||
+                    s->att2.ensure(Ts * att2 * s->esz) || s->head_i.ensure((2 * Ts * head_i + head_i + 1) * 4))))
+        return kr_fail(KR_ERR_HIP, "mixer scratch for %d tokens", T);
     for (SvRope& r : s->ropes) if (r.cs.ensure(Ts * (r.dims / 2) * 8)) return kr_fail(KR_ERR_HIP, "rope table");
     if (s->capture) { if (s->cap.ensure((size_t)c.n_layers * Ts * W * 4)) return kr_fail(KR_ERR_HIP, "capture buffer"); s->cap_T = T; }
     std::vector<int> nsplit(c.n_layers, 1);
     for (int li = 0; li < c.n_layers; li++) {
-        const kr_serve_layer& d = s->L[li].d;
-        nsplit[li] = kr_sv_attention_splits(T, d.heads, d.kv_heads, d.vdim, d.window > 0 ? std::min(max_pos + 1, d.window) : max_pos + 1);
-        if (nsplit[li] > 1 && (s->part_ml.ensure(Ts * d.heads * nsplit[li] * 8) || s->part_acc.ensure(Ts * d.heads * nsplit[li] * d.vdim * 4)))
+        const SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
+        const int visible = d.window > 0 ? std::min(max_pos + 1, d.window) : (d.chunk > 0 ? std::min(max_pos + 1, d.chunk) : max_pos + 1);
+        nsplit[li] = kr_sv_attention_splits(T, d.heads, l.att_heads_kv(), l.att_vdim(), visible);
+        if (nsplit[li] > 1 && (s->part_ml.ensure(Ts * d.heads * nsplit[li] * 8) || s->part_acc.ensure(Ts * d.heads * nsplit[li] * l.att_vdim() * 4)))
             return kr_fail(KR_ERR_HIP, "attention split scratch");
     }
     const bool want_amax = argmax_out != nullptr;
@@ -453,11 +580,11 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     float* x = (float*)s->x.p;
     {
         Timer tm(s, 7);
-        kr_sv_embed(s->embed.p, s->f32, d_tok, x, T, W, st);
+        kr_sv_embed(s->embed.p, s->f32, d_tok, x, c.pre_norm ? nullptr : s->h.p, T, W, st);     // without input norms the first sublayer reads the embedding row itself
     }
     {
         Timer tm(s, 2);
-        for (SvRope& r : s->ropes) kr_sv_rope_table(d_pos, (const double*)r.inv_freq.p, (float2*)r.cs.p, T, r.dims / 2, st);
+        for (SvRope& r : s->ropes) kr_sv_rope_table(d_pos, (const double*)r.inv_freq.p, (float2*)r.cs.p, T, r.dims / 2, r.mult, st);
     }
     int* mi = (int*)s->moe_i.p;
     // down projection of a gated feed-forward: decode-sized problems form the activation inside the projection's launch, larger ones write it once
@@ -467,26 +594,87 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         g.A = s->y.p; g.lda = F;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
     };
-    { Timer tm(s, 0); kr_sv_norm(x, nullptr, (const float*)s->L[0].norm_w.p, (const float*)s->L[0].norm_b.p, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, st); }
+    // the residual sum that ends a sublayer (or, in a parallel block, the layer); `next`: the norm of the sublayer that reads the new x, null with
+    // hand_on = the row as it is, or nothing when no sublayer follows
+    auto residual = [&](const float* mixp, const float* dense, const float* shared, const float* rows, const int* pair_pos, int top, const DevBuf* post_w, const DevBuf* post_b,
+                        bool hand_on, const DevBuf* next_w, const DevBuf* next_b) {
+        Timer tm(s, 6);
+        KrSvResidual r{};
+        r.x = x; r.mix = mixp; r.dense = dense; r.shared = shared; r.rows = rows; r.pair_pos = pair_pos; r.wts = (const float*)s->wts.p; r.top = top;
+        r.post_w = post_w ? (const float*)post_w->p : nullptr; r.post_b = (post_w && c.norm_bias && post_b) ? (const float*)post_b->p : nullptr; r.mult = c.residual_mult;
+        r.norm_w = (hand_on && next_w) ? (const float*)next_w->p : nullptr; r.norm_b = (hand_on && next_w && c.norm_bias && next_b) ? (const float*)next_b->p : nullptr;
+        r.h_out = hand_on ? s->h.p : nullptr; r.T = T; r.width = W; r.kind = c.norm_kind; r.eps = c.norm_eps;
+        kr_sv_residual_norm(r, s->f32, st);
+    };
+    if (c.pre_norm) { Timer tm(s, 0); kr_sv_norm(x, nullptr, (const float*)s->L[0].norm_w.p, c.norm_bias ? (const float*)s->L[0].norm_b.p : nullptr, s->h.p, s->f32, T, W, c.norm_eps, c.norm_kind, st); }
+    int head_rows_for = 0;               // the head row tables in head_i are valid for this head count
     for (int li = 0; li < c.n_layers; li++) {
         SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
-        float* hz = (float*)s->qkv.p;                    // [T, n_h]: q | k | v | router logits | gate | up of this layer
+        const SvLayer* nx = li + 1 < c.n_layers ? &s->L[li + 1] : nullptr;
+        const bool has_ff = d.mlp_kind != KR_SERVE_MLP_NONE;
+        float* hz = (float*)s->qkv.p;                    // [T, n_h]: q | k | v (or the latents) | router logits | gate | up of this layer
         KrSvGemm g{};
-        g.A = s->h.p; g.lda = W; g.W = l.hw.p; g.C = hz; g.ldc = l.n_h; g.M = T; g.N = l.n_h; g.K = W;
+        // a parallel block multiplies its one input by every matrix at once; a sequential block's feed-forward reads the x its mixer leaves
+        g.A = s->h.p; g.lda = W; g.W = l.hw.p; g.C = hz; g.ldc = l.n_h; g.M = T; g.N = seq ? l.n_qkv : l.n_h; g.K = W;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         const SvLayer& kvl = d.kv_from >= 0 ? s->L[d.kv_from] : l;
         KrSvAttn a{};
-        a.qkv = hz; a.ldq = l.n_h; a.heads = d.heads; a.kv_heads = d.kv_heads; a.dim = d.dim; a.vdim = d.vdim; a.rot_dims = d.rot_dims;
-        a.rot_interleaved = d.rot_interleaved; a.unit_norm = d.qk_unit_norm; a.own_kv = d.kv_from < 0; a.eps = c.norm_eps; a.scale = d.scale; a.window = d.window;
-        a.sink = d.has_sink ? (const float*)l.sink.p : nullptr; a.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
-        a.kpool = kvl.kpool.p; a.vpool = kvl.vpool.p; a.page_table = d_tab; a.table_ld = s->n_pages; a.slot = d_slot; a.pos = d_pos; a.page_tokens = PT; a.T = T;
+        a.heads = d.heads; a.kv_heads = l.att_heads_kv(); a.dim = l.att_dim(); a.vdim = l.att_vdim();
+        a.eps = c.norm_eps; a.scale = d.scale; a.window = d.window; a.chunk = d.chunk; a.slopes = d.dist_bias ? (const float*)l.slopes.p : nullptr;
+        a.sink = d.has_sink ? (const float*)l.sink.p : nullptr;
+        a.kpool = kvl.kpool.p; a.page_table = d_tab; a.table_ld = s->n_pages; a.slot = d_slot; a.pos = d_pos; a.page_tokens = PT; a.T = T;
         a.out = s->att.p;
         a.nsplit = nsplit[li]; a.part_ml = (float*)s->part_ml.p; a.part_acc = (float*)s->part_acc.p;
-        { Timer tm(s, 2); kr_sv_qk_prep(a, s->f32, st); }
-        { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
+        const void* o_in = s->att.p;
+        if (!l.latent()) {
+            a.qkv = hz; a.ldq = l.n_h; a.rot_dims = d.rot_dims; a.rot_interleaved = d.rot_interleaved; a.unit_norm = d.qk_unit_norm; a.own_kv = d.kv_from < 0;
+            a.q_norm_w = (const float*)l.q_norm.p; a.k_norm_w = (const float*)l.k_norm.p;
+            a.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr;
+            a.vpool = kvl.vpool.p; a.ldk = d.kv_heads * d.dim; a.ldv = d.kv_heads * d.vdim;
+            a.v_mix = d.v_mix; a.v_lambda = (const float*)l.vmix.p; a.v_first = (float*)s->v_first.p;
+            { Timer tm(s, 2); kr_sv_qk_prep(a, s->f32, st); }
+            { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
+        } else {
+            // queries: norm the latent, W_uq, turn the rotated part, fold W_uk of every head into the plain part; keys / values: the normed latent and the
+            // turned shared part are the cache row, read by the attention kernels as ONE key / value head whose values are the leading kv_rank of the key row
+            const int H = d.heads, R = d.kv_rank, De = l.att_dim();
+            KrSvLatent q{};
+            q.dz = hz; q.ld = l.n_h; q.q_rank = d.q_rank; q.kv_rank = R; q.rot = d.rot_dims; q.heads = H; q.dim = d.dim;
+            q.dq_norm_w = (const float*)l.dq_norm.p; q.dkv_norm_w = (const float*)l.dkv_norm.p; q.eps = c.norm_eps;
+            q.cs = d.rot_dims ? (const float2*)s->ropes[l.rope_id].cs.p : nullptr; q.cq = s->lq_c.p;
+            q.pool = l.kpool.p; q.page_table = d_tab; q.table_ld = s->n_pages; q.slot = d_slot; q.pos = d_pos; q.page_tokens = PT; q.T = T;
+            int* hseg = (int*)s->head_i.p; int* hrows = hseg + H + 1; int* hgroup = hrows + (size_t)T * H;
+            {
+                Timer tm(s, 2);
+                kr_sv_latent_prep(q, s->f32, st);
+                if (head_rows_for != H) { kr_sv_head_rows(T, H, hseg, hrows, hgroup, st); head_rows_for = H; }
+            }
+            g = KrSvGemm{}; g.A = s->lq_c.p; g.lda = d.q_rank; g.W = l.uq.p; g.C = (float*)s->lq_2.p; g.ldc = H * (d.dim + d.rot_dims); g.M = T; g.N = g.ldc; g.K = d.q_rank;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            { Timer tm(s, 2); kr_sv_latent_q(q, (const float*)s->lq_2.p, s->lq_n.p, (float*)s->lq_e.p, s->f32, st); }
+            g = KrSvGemm{}; g.A = s->lq_n.p; g.lda = d.dim; g.a_rows = hrows; g.W = l.ukT.p; g.w_stride = (size_t)R * d.dim; g.C = (float*)s->lq_e.p; g.ldc = De; g.c_rows = hrows;
+            g.M = T * H; g.N = R; g.K = d.dim; g.seg = hseg; g.row_group = hgroup; g.n_groups = H; g.rowwise_upto = 16 * H;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            a.qkv = (float*)s->lq_e.p; a.ldq = H * De; a.vpool = l.kpool.p; a.ldk = De; a.ldv = De;
+            { Timer tm(s, 3); kr_sv_attention(a, s->f32, st); }
+            g = KrSvGemm{}; g.A = s->att.p; g.lda = R; g.a_rows = hrows; g.W = l.uv.p; g.w_stride = (size_t)d.vdim * R; g.C = (float*)s->att2.p; g.ldc = d.vdim; g.c_rows = hrows; g.c_storage = 1;
+            g.M = T * H; g.N = d.vdim; g.K = R; g.seg = hseg; g.row_group = hgroup; g.n_groups = H; g.rowwise_upto = 16 * H;
+            { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+            o_in = s->att2.p;
+        }
         g = KrSvGemm{};
-        g.A = s->att.p; g.lda = d.heads * d.vdim; g.W = l.o.p; g.C = (float*)s->mix.p; g.ldc = W; g.M = T; g.N = W; g.K = d.heads * d.vdim;
+        g.A = o_in; g.lda = d.heads * d.vdim; g.W = l.o.p; g.C = (float*)s->mix.p; g.ldc = W; g.M = T; g.N = W; g.K = d.heads * d.vdim;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
+        if (seq) {
+            // the mixer's sublayer ends here; the new x, normed or as it is, is the feed-forward's input (or the next layer's when there is none)
+            if (has_ff) residual((const float*)s->mix.p, nullptr, nullptr, nullptr, nullptr, 0, c.post_norm ? &l.post1_w : nullptr, &l.post1_b, true, c.pre_norm ? &l.norm2_w : nullptr, &l.norm2_b);
+            else residual((const float*)s->mix.p, nullptr, nullptr, nullptr, nullptr, 0, c.post_norm ? &l.post1_w : nullptr, &l.post1_b, nx != nullptr, (nx && c.pre_norm) ? &nx->norm_w : nullptr,
+                          nx ? &nx->norm_b : nullptr);
+            if (has_ff && l.n_h > l.off_router) {
+                g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = (const char*)l.hw.p + (size_t)l.off_router * W * s->esz; g.C = hz + l.off_router; g.ldc = l.n_h; g.M = T; g.N = l.n_h - l.off_router; g.K = W;
+                Timer tm(s, 1); kr_sv_gemm(g, s->f32, st);
+            }
+        }
         const float *dense = nullptr, *shared = nullptr, *rows = nullptr; const int* pair_pos = nullptr;
         if (d.mlp_kind == KR_SERVE_MLP_DENSE) {
             g = KrSvGemm{}; g.W = l.down.p; g.C = (float*)s->ffout.p; g.ldc = W; g.M = T; g.N = W; g.K = d.ff;
@@ -497,7 +685,8 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
             int* counts_d = mi; int* seg = mi + E; int* cursor = seg + E + 1; int* src_row = cursor + E; int* row_group = src_row + P; int* pp = row_group + P;
             {
                 Timer tm(s, 4);
-                kr_sv_router_select(hz + l.off_router, l.n_h, s->f32 ? 1 : 2, T, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p, (float*)s->wts.p, st);
+                kr_sv_router_select(hz + l.off_router, l.n_h, s->f32 ? 1 : 2, d.router_bias ? (const float*)l.router_b.p : nullptr, T, E, top, d.groups, d.keep, d.renorm, (int*)s->ids.p,
+                                    (float*)s->wts.p, st);
                 kr_sv_moe_sort((const int*)s->ids.p, T, top, E, counts_d, seg, cursor, src_row, row_group, pp, st);
             }
             g = KrSvGemm{}; g.A = s->h.p; g.lda = W; g.W = l.egu.p; g.w_stride = (size_t)2 * F * W; g.C = (float*)s->gu.p; g.ldc = 2 * F; g.M = P; g.N = 2 * F; g.K = W;
@@ -514,16 +703,14 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
                 shared = (const float*)s->ffout.p;
             }
         }
-        {   // x += mixer + feed-forward, and the next layer's normed input from the same launch
-            Timer tm(s, 6);
-            const SvLayer* nx = li + 1 < c.n_layers ? &s->L[li + 1] : nullptr;
-            kr_sv_residual_norm(x, (const float*)s->mix.p, dense, shared, rows, pair_pos, (const float*)s->wts.p, d.top, T, W, nx ? (const float*)nx->norm_w.p : nullptr,
-                                nx ? (const float*)nx->norm_b.p : nullptr, s->h.p, s->f32, c.norm_eps, c.norm_kind, st);
-        }
+        // x += the layer's sublayers (parallel block) or the feed-forward alone (sequential), and the next layer's input from the same launch
+        if (!seq) residual((const float*)s->mix.p, dense, shared, rows, pair_pos, d.top, nullptr, nullptr, nx != nullptr, (nx && c.pre_norm) ? &nx->norm_w : nullptr, nx ? &nx->norm_b : nullptr);
+        else if (has_ff) residual(nullptr, dense, shared, rows, pair_pos, d.top, c.post_norm ? &l.post2_w : nullptr, &l.post2_b, nx != nullptr, (nx && c.pre_norm) ? &nx->norm_w : nullptr,
+                                  nx ? &nx->norm_b : nullptr);
         if (s->capture) KR_HIP(hipMemcpyAsync((float*)s->cap.p + (size_t)li * Ts * W, x, Ts * W * 4, hipMemcpyDeviceToDevice, st));
     }
     if (n_want > 0) {
-        { Timer tm(s, 0); kr_sv_norm(x, d_want, (const float*)s->fnorm_w.p, (const float*)s->fnorm_b.p, s->hw.p, s->f32, n_want, W, c.norm_eps, c.norm_kind, st); }
+        { Timer tm(s, 0); kr_sv_norm(x, d_want, (const float*)s->fnorm_w.p, c.norm_bias ? (const float*)s->fnorm_b.p : nullptr, s->hw.p, s->f32, n_want, W, c.norm_eps, c.norm_kind, st); }
         KrSvGemm g{}; g.A = s->hw.p; g.lda = W; g.W = s->head.p; g.C = (float*)s->logits.p; g.ldc = c.vocab; g.M = n_want; g.N = c.vocab; g.K = W;
         { Timer tm(s, 1); kr_sv_gemm(g, s->f32, st); }
         if (want_amax) { Timer tm(s, 7); kr_sv_argmax((const float*)s->logits.p, n_want, c.vocab, (int*)s->amax.p, st); }
@@ -540,7 +727,7 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
         mixin((uint64_t)T); mixin((uint64_t)n_want); mixin(want_amax);
         for (int v : nsplit) mixin((uint64_t)v);
         for (const DevBuf* b : {&s->meta, &s->x, &s->h, &s->qkv, &s->att, &s->mix, &s->gu, &s->y, &s->rows, &s->ffout, &s->ids, &s->wts, &s->rz, &s->moe_i, &s->hw, &s->logits,
-                                &s->amax, &s->part_ml, &s->part_acc}) mixin((uint64_t)(uintptr_t)b->p);
+                                &s->amax, &s->part_ml, &s->part_acc, &s->v_first, &s->lq_c, &s->lq_2, &s->lq_n, &s->lq_e, &s->att2, &s->head_i}) mixin((uint64_t)(uintptr_t)b->p);
         for (const SvRope& r : s->ropes) mixin((uint64_t)(uintptr_t)r.cs.p);
         hipGraphExec_t exec = nullptr;
         for (auto& g : s->graphs) if (g.key == key) exec = g.exec;

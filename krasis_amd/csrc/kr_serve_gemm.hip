@@ -19,6 +19,13 @@ typedef uint32_t gu4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float gm_ld(const float* p) { return *p; }
 __device__ __forceinline__ float gm_ld(const uint16_t* p) { return kr_bf16_to_f32(*p); }
+// one element of C: f32, or the storage type when the output feeds another GEMM as it is (BF = a bf16 store)
+template <bool BF>
+__device__ __forceinline__ void gm_store(const KrSvGemm& g, int m, int n, float v) {
+    const size_t i = (size_t)(g.c_rows ? g.c_rows[m] : m) * g.ldc + n;
+    if (BF && g.c_storage) ((uint16_t*)g.C)[i] = kr_f32_to_bf16(v);
+    else g.C[i] = v;
+}
 
 // row tile `tile` of a grouped problem: walks the segment table; returns false past the last tile
 __device__ __forceinline__ bool gm_find_tile(const int* seg, int n_groups, int tile, int BM, int& group, int& m0, int& mend) {
@@ -136,7 +143,7 @@ __global__ void __launch_bounds__(256) sv_gemv_kernel(const KrSvGemm g, int mbas
             float v = acc[m][c];
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-            if (lane == 0 && m < mcnt && n0 + c < g.N) g.C[(size_t)(m0 + m) * g.ldc + n0 + c] = v;
+            if (lane == 0 && m < mcnt && n0 + c < g.N) gm_store<sizeof(T) == 2>(g, m0 + m, n0 + c, v);
         }
 }
 
@@ -187,7 +194,7 @@ __global__ void __launch_bounds__(256) sv_gemm_f32_kernel(const KrSvGemm g) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int n = n0 + tx * 4 + j;
-            if (n < g.N) g.C[(size_t)m * g.ldc + n] = acc[i][j];
+            if (n < g.N) gm_store<false>(g, m, n, acc[i][j]);
         }
     }
 }
@@ -280,7 +287,7 @@ __global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int m = m0 + wr * (BM / 2) + a * 32 + (i & 3) + 8 * (i >> 2) + 4 * h;
-                if (m < mend) g.C[(size_t)m * g.ldc + n] = acc[a][b][i];
+                if (m < mend) gm_store<true>(g, m, n, acc[a][b][i]);
             }
         }
 }
@@ -288,7 +295,7 @@ __global__ void __launch_bounds__(256) sv_gemm_bf16_kernel(const KrSvGemm g) {
 
 bool kr_sv_gemm_small(const KrSvGemm& g) {
     // decode-sized problems: a pass over the weights per 8 rows; grouped problems take one row per workgroup row (each row has its own expert)
-    return g.seg ? (g.M <= 64 && g.row_group) : g.M <= 16;
+    return g.seg ? (g.M <= (g.rowwise_upto > 64 ? g.rowwise_upto : 64) && g.row_group) : g.M <= 16;
 }
 
 void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st) {

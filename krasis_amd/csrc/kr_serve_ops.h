@@ -21,6 +21,9 @@ struct KrSvGemm {
     // small-M form only (kr_sv_gemm_small): A is not read but formed on the fly as the gated activation of act_gu [M, act_ld] f32 (gate at column k, up at
     // column K + k), rounded to the storage type -- the down projection of a feed-forward without a launch and a buffer for the activation
     const float* act_gu; int act_ld, act_kind; float act_limit, act_alpha;
+    const int* c_rows;               // optional: problem row r writes C row c_rows[r] (a grouped problem whose rows return to their own order)
+    int c_storage;                   // != 0: C holds the storage type (bf16 in a bf16 store) instead of f32 -- the output feeds another GEMM as it is
+    int rowwise_upto;                // grouped problems: the wave-per-column form up to this many rows (0 = the default of 64)
 };
 void kr_sv_gemm(const KrSvGemm& g, bool f32, hipStream_t st);
 bool kr_sv_gemm_small(const KrSvGemm& g);      // true: kr_sv_gemm takes the wave-per-column form for this problem (and honours act_gu)
@@ -28,20 +31,26 @@ bool kr_sv_gemm_small(const KrSvGemm& g);      // true: kr_sv_gemm takes the wav
 enum { KR_SV_NORM_LAYER = 0, KR_SV_NORM_RMS = 1 };
 enum { KR_SV_ACT_GELU_TANH = 0, KR_SV_ACT_CLAMPED_SWIGLU = 1, KR_SV_ACT_SILU = 2 };
 
-void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, int T, int width, hipStream_t st);
+// x[t] = table[tokens[t]]; with h_out also the row in the storage type (the first sublayer's input in a design without input norms)
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, hipStream_t st);
 // out[r] = norm(x[rows ? rows[r] : r]) * w (+ b): two passes over the row, f32; out in the storage type
 void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, hipStream_t st);
-// cos / sin of pos * inv_freq for every token of the step: cs[t][i] = (cos, sin), the angle formed in double
-void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, hipStream_t st);
+// cos / sin of pos * inv_freq for every token of the step: cs[t][i] = mult * (cos, sin), the angle formed in double
+void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, float mult, hipStream_t st);
 
 struct KrSvAttn {
     float* qkv; int ldq;             // [T, ldq] f32: q heads, then k heads, then v heads (k / v absent when the layer borrows another layer's cache)
     int heads, kv_heads, dim, vdim, rot_dims, rot_interleaved, unit_norm, own_kv;
+    const float* q_norm_w; const float* k_norm_w;   // [dim] each: unit_norm == 2 (weighted, before the rotation)
     float eps, scale;
     int window;                      // 0 = every earlier position
+    int chunk;                       // > 0: only the keys of the query's own block of `chunk` positions (counted from position 0 of the request)
+    const float* slopes;             // [heads] or null: score -= slopes[h] * (query position - key position)
+    int v_mix; const float* v_lambda; float* v_first;   // 1: values also kept in v_first [T, kv_heads * vdim]; 2: v <- (1 - *v_lambda) v + *v_lambda v_first
     const float* sink;               // [heads] or null
     const float2* cs;                // rope table of the step for this layer's rotation
-    void* kpool; void* vpool;        // [pages][page_tokens][kv_heads * dim | vdim] storage type
+    void* kpool; void* vpool;        // [pages][page_tokens][ldk | ldv] storage type; head g at g * dim | g * vdim of a row (vpool may be kpool: values that are a
+    int ldk, ldv;                    //   leading part of the key row)
     const int* page_table; int table_ld;   // [slots][table_ld]
     const int* slot; const int* pos; // per token
     int page_tokens, T;
@@ -59,15 +68,39 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed
 // `groups` groups (a group's score = its largest), `top` experts among them; weights = the softmax scores (renorm != 0: divided by their sum).
 // The logits come from kr_sv_gemm: an f32 store multiplies by the f32 gate; a bf16 store by the gate as two bf16 terms (hi + lo rows), which
 // carries 16 bits of the gate's mantissa through the matrix cores.
-void kr_sv_router_select(const float* z, int ld, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st);
+// bias [E] or null joins the logits before anything else.
+void kr_sv_router_select(const float* z, int ld, int parts, const float* bias, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st);
 // rows of every expert: seg[E + 1], src_row[T * top] (token of sorted row), row_group[T * top], pair_pos[T * top] (sorted row of (token, slot))
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st);
 // gu rows `ld` floats apart (gate at [0, F), up at [F, 2F)) -> y [M, F] storage type
 void kr_sv_act(const float* gu, int ld, void* y, bool f32, int M, int F, int kind, float limit, float alpha, hipStream_t st);
-// x[t] += mix[t] + (dense[t] + shared[t] + sum_s wts[t][s] * rows[pair_pos[t][s]]); null terms are skipped.  With norm_w the normed row of the NEW x
-// (the next layer's input) is written to h_out in the storage type by the same launch.
-void kr_sv_residual_norm(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
-                         int width, const float* norm_w, const float* norm_b, void* h_out, bool out_f32, float eps, int kind, hipStream_t st);
+// y[t] = mix[t] + (dense[t] + shared[t] + sum_s wts[t][s] * rows[pair_pos[t][s]]) (null terms are skipped); with post_w, y <- norm(y) * post_w (+ post_b);
+// x[t] += mult * y[t].  With h_out the NEW row goes there in the storage type by the same launch: normed with norm_w (+ norm_b) -- the next sublayer's
+// input -- or, without norm_w, as it is.
+struct KrSvResidual {
+    float* x; const float* mix; const float* dense; const float* shared; const float* rows; const int* pair_pos; const float* wts; int top;
+    const float* post_w; const float* post_b; float mult;
+    const float* norm_w; const float* norm_b; void* h_out;
+    int T, width, kind; float eps;
+};
+void kr_sv_residual_norm(const KrSvResidual& r, bool out_f32, hipStream_t st);
+
+// ---- latent mixer (queries and keys / values through low-rank latents; the cache row is [latent | rotated shared key part])
+struct KrSvLatent {
+    const float* dz; int ld;         // [T, ld] f32: W_dq h [q_rank] | W_dkv h [kv_rank + rot]
+    int q_rank, kv_rank, rot, heads, dim;
+    const float* dq_norm_w; const float* dkv_norm_w; float eps;
+    const float2* cs;                // rotation table of the step [T, rot / 2]
+    void* cq;                        // out [T, q_rank] storage type: rms(W_dq h) * w
+    void* pool; const int* page_table; int table_ld; const int* slot; const int* pos; int page_tokens, T;    // cache rows [kv_rank + rot] storage type
+};
+// normed query latent -> cq; normed key / value latent and the rotated shared key part -> the cache row of (slot, position)
+void kr_sv_latent_prep(const KrSvLatent& a, bool f32, hipStream_t st);
+// q2 [T, heads, dim + rot] f32 (W_uq c_q): the plain part -> qn [T, heads, dim] storage type (to be folded into the latent space by a GEMM), the rotated
+// part, turned, -> qe [T, heads, kv_rank + rot] f32 at column kv_rank
+void kr_sv_latent_q(const KrSvLatent& a, const float* q2, void* qn, float* qe, bool f32, hipStream_t st);
+// rows of a problem grouped by head over [T, heads, *] arrays: seg[h] = h * T, rows[h * T + t] = t * heads + h, group[h * T + t] = h
+void kr_sv_head_rows(int T, int heads, int* seg, int* rows, int* group, hipStream_t st);
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st);
 // uniform values in [-amp, amp) from a counter hash of (seed, element); amp = 0 writes zeros
 void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, hipStream_t st);

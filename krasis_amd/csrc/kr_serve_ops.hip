@@ -46,10 +46,13 @@ __device__ __forceinline__ float sv_block_sum(float v, float* red) {
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, int width) {
+__global__ void __launch_bounds__(256) sv_embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, T* __restrict__ h_out, int width) {
     const int t = blockIdx.x;
     const T* row = table + (size_t)tokens[t] * width;
-    for (int c = threadIdx.x; c < width; c += 256) x[(size_t)t * width + c] = sv_ld(row + c);
+    for (int c = threadIdx.x; c < width; c += 256) {
+        x[(size_t)t * width + c] = sv_ld(row + c);
+        if (h_out) h_out[(size_t)t * width + c] = row[c];
+    }
 }
 
 template <typename T, int KIND>
@@ -75,12 +78,12 @@ __global__ void __launch_bounds__(256) sv_norm_kernel(const float* __restrict__ 
     }
 }
 
-__global__ void sv_rope_table_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq, float2* __restrict__ cs, int T, int half) {
+__global__ void sv_rope_table_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq, float2* __restrict__ cs, int T, int half, float mult) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= T * half) return;
     const int t = i / half, j = i - t * half;
     const double a = (double)pos[t] * inv_freq[j];
-    cs[i] = make_float2((float)cos(a), (float)sin(a));
+    cs[i] = make_float2((float)cos(a) * mult, (float)sin(a) * mult);
 }
 
 // one wave per (token, head): the head vector is staged in LDS, rotated and normed there; q heads are written back in place, k heads go to the
@@ -97,16 +100,32 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
         const size_t page = (size_t)a.page_table[(size_t)sl * a.table_ld + p / a.page_tokens];
         prow = page * a.page_tokens + (p % a.page_tokens);
     }
-    if (hh >= H + G) {                       // value head: copy
+    if (hh >= H + G) {                       // value head: copy, or blend with the values an earlier layer formed for this token
         const int g = hh - H - G;
         const float* v = row + (size_t)H * a.dim + (size_t)G * a.dim + (size_t)g * a.vdim;
-        T* dst = (T*)a.vpool + (prow * G + g) * a.vdim;
-        for (int d = lane; d < a.vdim; d += 64) sv_st(dst + d, v[d]);
+        T* dst = (T*)a.vpool + prow * a.ldv + (size_t)g * a.vdim;
+        float* vf = a.v_mix ? a.v_first + ((size_t)t * G + g) * a.vdim : nullptr;
+        const float lam = a.v_mix == 2 ? *a.v_lambda : 0.0f;
+        for (int d = lane; d < a.vdim; d += 64) {
+            float val = v[d];
+            if (a.v_mix == 1) vf[d] = val;
+            else if (a.v_mix == 2) val = (1.0f - lam) * val + lam * vf[d];
+            sv_st(dst + d, val);
+        }
         return;
     }
     float* v = row + (size_t)hh * a.dim;
     for (int d = lane; d < a.dim; d += 64) hv[d] = v[d];
     __syncthreads();
+    if (a.unit_norm == 2) {                  // weighted, before the rotation
+        const float* w = hh < H ? a.q_norm_w : a.k_norm_w;
+        float s2 = 0.0f;
+        for (int d = lane; d < a.dim; d += 64) s2 = __builtin_fmaf(hv[d], hv[d], s2);
+        s2 = sv_wave_sum(s2);
+        const float inv2 = 1.0f / sqrtf(s2 / (float)a.dim + a.eps);
+        for (int d = lane; d < a.dim; d += 64) hv[d] = hv[d] * inv2 * w[d];
+        __syncthreads();
+    }
     const int half = a.rot_dims / 2;
     const float2* cs = a.cs + (size_t)t * half;
     float ss = 0.0f;
@@ -120,13 +139,13 @@ __global__ void __launch_bounds__(64) sv_qk_prep_kernel(const KrSvAttn a) {
     }
     for (int d = a.rot_dims + lane; d < a.dim; d += 64) ss = __builtin_fmaf(hv[d], hv[d], ss);
     ss = sv_wave_sum(ss);
-    const float inv = a.unit_norm ? 1.0f / sqrtf(ss / (float)a.dim + a.eps) : 1.0f;
+    const float inv = a.unit_norm == 1 ? 1.0f / sqrtf(ss / (float)a.dim + a.eps) : 1.0f;
     __syncthreads();
     if (hh < H) {
         for (int d = lane; d < a.dim; d += 64) v[d] = hv[d] * inv;
     } else {
         const int g = hh - H;
-        T* dst = (T*)a.kpool + (prow * G + g) * a.dim;
+        T* dst = (T*)a.kpool + prow * a.ldk + (size_t)g * a.dim;
         for (int d = lane; d < a.dim; d += 64) sv_st(dst + d, hv[d] * inv);
     }
 }
@@ -164,7 +183,10 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
     for (int i = tid; i < RM * dim; i += 256) qs[i] = i < nr * dim ? q[i] * a.scale : 0.0f;
     __syncthreads();
     SV_STAMP(1);
-    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    const int lo = a.window > 0 ? max(0, p - a.window + 1) : (a.chunk > 0 ? p - p % a.chunk : 0);
+    float slope[RM];
+#pragma unroll
+    for (int r = 0; r < RM; r++) slope[r] = (a.slopes && r < nr) ? a.slopes[h0 + r] : 0.0f;
     float m[RM], l[RM], acc[RM][VC];
 #pragma unroll
     for (int r = 0; r < RM; r++) {
@@ -173,7 +195,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         for (int c = 0; c < VC; c++) acc[r][c] = 0.0f;
     }
     const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
-    const bool vec = ((size_t)dim * sizeof(T)) % 16 == 0;
+    const bool vec = ((size_t)dim * sizeof(T)) % 16 == 0 && ((size_t)a.ldk * sizeof(T)) % 16 == 0;
     const int npiece = dim / VEC;
     auto widen = [](const sv_u4& kv, float* kf) {
         if constexpr (sizeof(T) == 2) {
@@ -193,7 +215,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         const bool live = j <= p;
         const int jc = min(j, p);                            // lanes past the last key score it again; their weight is set to 0
         const int prow = table[jc / a.page_tokens] * a.page_tokens + (jc % a.page_tokens);
-        const T* k = kp + ((size_t)prow * G + g) * dim;
+        const T* k = kp + (size_t)prow * a.ldk + (size_t)g * dim;
         constexpr int U = 16 / VC;                           // keys whose value rows are requested together
         const int nk = min(64, p - j0 + 1);
         float va[U][VC], vb[U][VC];
@@ -201,7 +223,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int pr = __builtin_amdgcn_readlane(prow, min(jb + u, 63));
-                const T* vr = vp + ((size_t)pr * G + g) * vdim;
+                const T* vr = vp + (size_t)pr * a.ldv + (size_t)g * vdim;
 #pragma unroll
                 for (int c = 0; c < VC; c++) { const int d = lane + 64 * c; vv[u][c] = d < vdim ? sv_ld(vr + d) : 0.0f; }
             }
@@ -257,7 +279,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
         SV_STAMP(3);
 #pragma unroll
         for (int r = 0; r < RM; r++) {
-            const float sr = live ? s[r] : -INFINITY;
+            const float sr = live ? s[r] - slope[r] * (float)(p - j) : -INFINITY;
             const float mn = fmaxf(m[r], sv_wave_max(sr));
             const float alpha = expf(m[r] - mn);               // first block of this wave: exp(-inf) = 0
             const float pj = live ? expf(sr - mn) : 0.0f;
@@ -388,8 +410,9 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
         while (end < TQ && t0 + end < a.T && a.slot[t0 + end] == sl && a.pos[t0 + end] == p0 + (end - base)) end++;
         const bool rv = tq_row >= base && tq_row < end;
         const int p_row = rv ? p0 + (tq_row - base) : -1;
-        const int lo_row = a.window > 0 ? max(0, p_row - a.window + 1) : 0;
-        const int hi = p0 + (end - base - 1), lo = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
+        const int lo_row = a.window > 0 ? max(0, p_row - a.window + 1) : (a.chunk > 0 && rv ? p_row - p_row % a.chunk : 0);
+        const int hi = p0 + (end - base - 1), lo = a.window > 0 ? max(0, p0 - a.window + 1) : (a.chunk > 0 ? p0 - p0 % a.chunk : 0);
+        const float slope_row = (a.slopes && rv) ? a.slopes[h_row] : 0.0f;
         const int* table = a.page_table + (size_t)sl * a.table_ld;
         float q[DQ];
         {
@@ -414,7 +437,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             }
 #pragma unroll
             for (int kb = 0; kb < 4; kb++) {
-                const T* k = kp + ((size_t)prow[kb] * G + g) * dim + qd * DQ;
+                const T* k = kp + (size_t)prow[kb] * a.ldk + (size_t)g * dim + qd * DQ;
                 sv_u4 kv[DQ / VEC];
 #pragma unroll
                 for (int u = 0; u < DQ / VEC; u++) kv[u] = *reinterpret_cast<const sv_u4*>(k + u * VEC);
@@ -442,7 +465,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
                 for (int i = 0; i < 4; i++) {
                     const int key = j0 + kb * 16 + 4 * qd + i;
                     const bool ok = rv && key <= p_row && key >= lo_row;
-                    st[kb][i] = ok ? st[kb][i] : -INFINITY;
+                    st[kb][i] = ok ? st[kb][i] - slope_row * (float)(p_row - key) : -INFINITY;
                     cm = fmaxf(cm, st[kb][i]);
                 }
             cm = fmaxf(cm, __shfl_xor(cm, 16)); cm = fmaxf(cm, __shfl_xor(cm, 32));
@@ -464,7 +487,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int pr = __shfl(prow[kb], 4 * qd + i);
-                    const T* vr = vp + ((size_t)pr * G + g) * vdim + row * DB;
+                    const T* vr = vp + (size_t)pr * a.ldv + (size_t)g * vdim + row * DB;
                     if constexpr ((DB * sizeof(T)) % 16 == 0) {
 #pragma unroll
                         for (int u = 0; u < DB / VEC; u++) {
@@ -551,12 +574,16 @@ __global__ void __launch_bounds__(64) sv_attn_merge_kernel(const KrSvAttn a) {
 
 // selection: one wave per token; the scores of the E experts live in LDS
 // z holds the logits as `parts` column blocks of E that are added (a gate stored as two bf16 terms gives two)
-__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int ld, int parts, int E, int top, int groups, int keep, int renorm,
-                                                              int* __restrict__ ids, float* __restrict__ wts) {
+__global__ void __launch_bounds__(64) sv_router_select_kernel(const float* __restrict__ z, int ld, int parts, const float* __restrict__ bias, int E, int top, int groups,
+                                                              int keep, int renorm, int* __restrict__ ids, float* __restrict__ wts) {
     extern __shared__ float lds[];           // s[E] | gscore[groups] | allowed flags as floats [groups]
     float* s = lds; float* gs = lds + E; float* gok = gs + groups;
     const int t = blockIdx.x, lane = threadIdx.x;
-    for (int e = lane; e < E; e += 64) { float v = z[(size_t)t * ld + e]; for (int q = 1; q < parts; q++) v += z[(size_t)t * ld + (size_t)q * E + e]; s[e] = v; }
+    for (int e = lane; e < E; e += 64) {
+        float v = z[(size_t)t * ld + e];
+        for (int q = 1; q < parts; q++) v += z[(size_t)t * ld + (size_t)q * E + e];
+        s[e] = bias ? v + bias[e] : v;
+    }
     __syncthreads();
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
@@ -675,18 +702,19 @@ __global__ void sv_act_kernel(const float* __restrict__ gu, int ld, T* __restric
     sv_st(y + i, v);
 }
 
-// one workgroup per token: the new residual row is formed in LDS, written back, and (with norm_w) normed from there for the next layer
+// one workgroup per token: the sublayers' output row is formed in LDS, normed there when the design norms sublayer outputs, added to the residual row,
+// and the new row is written back and handed on in the storage type -- normed for the next sublayer (norm_w) or as it is
 template <typename T, int KIND>
-__global__ void __launch_bounds__(256) sv_residual_norm_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ dense,
-                                                               const float* __restrict__ shared, const float* __restrict__ rows, const int* __restrict__ pair_pos,
-                                                               const float* __restrict__ wts, int top, int width, const float* __restrict__ norm_w,
-                                                               const float* __restrict__ norm_b, T* __restrict__ h_out, float eps) {
+__global__ void __launch_bounds__(256) sv_residual_norm_kernel(const KrSvResidual a, T* __restrict__ h_out) {
     extern __shared__ float xr[];            // [width]
     __shared__ float red[4];
     __shared__ int pp_s[64]; __shared__ float w_s[64];      // the token's expert rows and weights, read once (top <= 64; more fall back to global reads)
     const size_t t = blockIdx.x;
+    const int width = a.width, top = a.top;
+    const float* __restrict__ rows = a.rows; const float* __restrict__ mix = a.mix; const float* __restrict__ dense = a.dense; const float* __restrict__ shared = a.shared;
+    float* __restrict__ x = a.x;
     const bool staged = rows && top <= 64;
-    if (staged && threadIdx.x < top) { pp_s[threadIdx.x] = pair_pos[t * top + threadIdx.x]; w_s[threadIdx.x] = wts[t * top + threadIdx.x]; }
+    if (staged && threadIdx.x < top) { pp_s[threadIdx.x] = a.pair_pos[t * top + threadIdx.x]; w_s[threadIdx.x] = a.wts[t * top + threadIdx.x]; }
     if (rows) __syncthreads();
     float s1 = 0.0f;
     for (int c = threadIdx.x; c < width; c += 256) {
@@ -697,7 +725,7 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(float* __restrict
 #pragma unroll 4
                 for (int s = 0; s < top; s++) ff = __builtin_fmaf(w_s[s], rows[(size_t)pp_s[s] * width + c], ff);
             } else {
-                for (int s = 0; s < top; s++) ff = __builtin_fmaf(wts[t * top + s], rows[(size_t)pair_pos[t * top + s] * width + c], ff);
+                for (int s = 0; s < top; s++) ff = __builtin_fmaf(a.wts[t * top + s], rows[(size_t)a.pair_pos[t * top + s] * width + c], ff);
             }
             any = true;
         }
@@ -705,20 +733,91 @@ __global__ void __launch_bounds__(256) sv_residual_norm_kernel(float* __restrict
         if (dense) { ff = any ? ff + dense[i] : dense[i]; any = true; }
         float d = mix ? mix[i] : 0.0f;
         if (any) d = mix ? d + ff : ff;
-        const float v = x[i] + d;
+        if (a.post_w) { xr[c] = d; s1 += d; continue; }      // the sum waits for its norm
+        const float v = x[i] + a.mult * d;
         x[i] = v; xr[c] = v; s1 += v;
     }
-    if (!norm_w) return;
+    if (a.post_w) {
+        float mean = 0.0f;
+        if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
+        float q = 0.0f;
+        for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }
+        const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
+        s1 = 0.0f;
+        for (int c = threadIdx.x; c < width; c += 256) {
+            const size_t i = t * width + c;
+            float y = (xr[c] - mean) * inv * a.post_w[c];
+            if (a.post_b) y += a.post_b[c];
+            const float v = x[i] + a.mult * y;
+            x[i] = v; xr[c] = v; s1 += v;
+        }
+    }
+    if (!h_out) return;
+    if (!a.norm_w) {
+        for (int c = threadIdx.x; c < width; c += 256) sv_st(h_out + t * width + c, xr[c]);
+        return;
+    }
     float mean = 0.0f;
     if constexpr (KIND == KR_SV_NORM_LAYER) mean = sv_block_sum<4>(s1, red) / (float)width;
     float q = 0.0f;
     for (int c = threadIdx.x; c < width; c += 256) { const float dv = xr[c] - mean; q = __builtin_fmaf(dv, dv, q); }      // a thread re-reads its own columns
-    const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + eps);
+    const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)width + a.eps);
     for (int c = threadIdx.x; c < width; c += 256) {
-        float v = (xr[c] - mean) * inv * norm_w[c];
-        if (norm_b) v += norm_b[c];
+        float v = (xr[c] - mean) * inv * a.norm_w[c];
+        if (a.norm_b) v += a.norm_b[c];
         sv_st(h_out + t * width + c, v);
     }
+}
+
+// ---- latent mixer
+// one workgroup per (token, part): part 0 norms the query latent, part 1 norms the key / value latent into the cache row and turns the shared key part
+template <typename T>
+__global__ void __launch_bounds__(256) sv_latent_prep_kernel(const KrSvLatent a) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, part = blockIdx.y;
+    const float* z = a.dz + (size_t)t * a.ld + (part ? a.q_rank : 0);
+    const int n = part ? a.kv_rank : a.q_rank;
+    const float* w = part ? a.dkv_norm_w : a.dq_norm_w;
+    T* dst;
+    if (part) {
+        const int p = a.pos[t];
+        const size_t page = (size_t)a.page_table[(size_t)a.slot[t] * a.table_ld + p / a.page_tokens];
+        dst = (T*)a.pool + (page * a.page_tokens + (p % a.page_tokens)) * (size_t)(a.kv_rank + a.rot);
+    } else dst = (T*)a.cq + (size_t)t * a.q_rank;
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < n; c += 256) q = __builtin_fmaf(z[c], z[c], q);
+    const float inv = 1.0f / sqrtf(sv_block_sum<4>(q, red) / (float)n + a.eps);
+    for (int c = threadIdx.x; c < n; c += 256) sv_st(dst + c, z[c] * inv * w[c]);
+    if (part) {
+        const float2* cs = a.cs + (size_t)t * (a.rot / 2);
+        for (int i = threadIdx.x; i < a.rot / 2; i += 256) {
+            const float u = z[n + 2 * i], v = z[n + 2 * i + 1];
+            const float2 c = cs[i];
+            sv_st(dst + n + 2 * i, u * c.x - v * c.y); sv_st(dst + n + 2 * i + 1, v * c.x + u * c.y);
+        }
+    }
+}
+// one wave per (token, head)
+template <typename T>
+__global__ void __launch_bounds__(64) sv_latent_q_kernel(const KrSvLatent a, const float* __restrict__ q2, T* __restrict__ qn, float* __restrict__ qe) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* q = q2 + ((size_t)t * a.heads + h) * (a.dim + a.rot);
+    T* n = qn + ((size_t)t * a.heads + h) * a.dim;
+    for (int d = lane; d < a.dim; d += 64) sv_st(n + d, q[d]);
+    float* e = qe + ((size_t)t * a.heads + h) * (a.kv_rank + a.rot) + a.kv_rank;
+    const float2* cs = a.cs + (size_t)t * (a.rot / 2);
+    for (int i = lane; i < a.rot / 2; i += 64) {
+        const float u = q[a.dim + 2 * i], v = q[a.dim + 2 * i + 1];
+        const float2 c = cs[i];
+        e[2 * i] = u * c.x - v * c.y; e[2 * i + 1] = v * c.x + u * c.y;
+    }
+}
+__global__ void sv_head_rows_kernel(int T, int heads, int* __restrict__ seg, int* __restrict__ rows, int* __restrict__ group) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i <= heads) seg[i] = i * T;
+    if (i >= T * heads) return;
+    const int h = i / T, t = i - h * T;
+    rows[i] = t * heads + h; group[i] = h;
 }
 
 __global__ void __launch_bounds__(1024) sv_argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out) {
@@ -757,10 +856,10 @@ void kr_sv_fill_uniform(void* p, bool f32, size_t n, uint64_t seed, float amp, h
     else hipLaunchKernelGGL(sv_fill_uniform_kernel<uint16_t>, grid, dim3(256), 0, st, (uint16_t*)p, n, seed, amp);
 }
 
-void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, int T, int width, hipStream_t st) {
+void kr_sv_embed(const void* table, bool f32, const int* tokens, float* x, void* h_out, int T, int width, hipStream_t st) {
     if (T <= 0) return;
-    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, width);
-    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, width);
+    if (f32) hipLaunchKernelGGL(sv_embed_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)table, tokens, x, (float*)h_out, width);
+    else hipLaunchKernelGGL(sv_embed_kernel<uint16_t>, dim3(T), dim3(256), 0, st, (const uint16_t*)table, tokens, x, (uint16_t*)h_out, width);
 }
 
 void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b, void* out, bool out_f32, int R, int width, float eps, int kind, hipStream_t st) {
@@ -771,10 +870,10 @@ void kr_sv_norm(const float* x, const int* rows, const float* w, const float* b,
 #undef SV_NORM
 }
 
-void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, hipStream_t st) {
+void kr_sv_rope_table(const int* pos, const double* inv_freq, float2* cs, int T, int half, float mult, hipStream_t st) {
     const int n = T * half;
     if (n <= 0) return;
-    hipLaunchKernelGGL(sv_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, st, pos, inv_freq, cs, T, half);
+    hipLaunchKernelGGL(sv_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, st, pos, inv_freq, cs, T, half, mult);
 }
 
 void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st) {
@@ -804,7 +903,7 @@ static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
     constexpr int VEC = 16 / sizeof(T);
     const int R = a.heads / a.kv_heads;
     if (!((R <= 16 && 16 % R == 0) || R % 16 == 0)) return false;
-    if (a.dim % (4 * VEC) != 0 || a.vdim % 16 != 0) return false;
+    if (a.dim % (4 * VEC) != 0 || a.vdim % 16 != 0 || a.ldk % VEC != 0 || a.ldv % VEC != 0) return false;
     const int Rb = R < 16 ? R : 16;
     KrSvAttn b = a;
     b.tq = a.nsplit > 1 ? 1 : 16 / Rb;      // a split launch is a decode-shaped step: its tokens belong to different requests
@@ -859,10 +958,10 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
 #undef SV_ATT
 }
 
-void kr_sv_router_select(const float* z, int ld, int parts, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st) {
+void kr_sv_router_select(const float* z, int ld, int parts, const float* bias, int T, int E, int top, int groups, int keep, int renorm, int* ids, float* wts, hipStream_t st) {
     if (T <= 0) return;
     const size_t lds = (size_t)(E + 2 * groups) * sizeof(float);
-    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, ld, parts, E, top, groups, keep, renorm, ids, wts);
+    hipLaunchKernelGGL(sv_router_select_kernel, dim3(T), dim3(64), lds, st, z, ld, parts, bias, E, top, groups, keep, renorm, ids, wts);
 }
 
 void kr_sv_moe_sort(const int* ids, int T, int top, int E, int* counts, int* seg, int* cursor, int* src_row, int* row_group, int* pair_pos, hipStream_t st) {
@@ -886,14 +985,29 @@ void kr_sv_act(const float* gu, int ld, void* y, bool f32, int M, int F, int kin
     else hipLaunchKernelGGL(sv_act_kernel<uint16_t>, grid, dim3(256), 0, st, gu, ld, (uint16_t*)y, M, F, kind, limit, alpha);
 }
 
-void kr_sv_residual_norm(float* x, const float* mix, const float* dense, const float* shared, const float* rows, const int* pair_pos, const float* wts, int top, int T,
-                         int width, const float* norm_w, const float* norm_b, void* h_out, bool out_f32, float eps, int kind, hipStream_t st) {
-    if (T <= 0) return;
-    const size_t lds = (size_t)width * sizeof(float);
-#define SV_RN(T_, K_) hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_>), dim3(T), dim3(256), lds, st, x, mix, dense, shared, rows, pair_pos, wts, top, width, norm_w, norm_b, (T_*)h_out, eps)
-    if (kind == KR_SV_NORM_LAYER) { if (out_f32) SV_RN(float, KR_SV_NORM_LAYER); else SV_RN(uint16_t, KR_SV_NORM_LAYER); }
+void kr_sv_residual_norm(const KrSvResidual& r, bool out_f32, hipStream_t st) {
+    if (r.T <= 0) return;
+    const size_t lds = (size_t)r.width * sizeof(float);
+#define SV_RN(T_, K_) hipLaunchKernelGGL((sv_residual_norm_kernel<T_, K_>), dim3(r.T), dim3(256), lds, st, r, (T_*)r.h_out)
+    if (r.kind == KR_SV_NORM_LAYER) { if (out_f32) SV_RN(float, KR_SV_NORM_LAYER); else SV_RN(uint16_t, KR_SV_NORM_LAYER); }
     else { if (out_f32) SV_RN(float, KR_SV_NORM_RMS); else SV_RN(uint16_t, KR_SV_NORM_RMS); }
 #undef SV_RN
+}
+
+void kr_sv_latent_prep(const KrSvLatent& a, bool f32, hipStream_t st) {
+    if (a.T <= 0) return;
+    if (f32) hipLaunchKernelGGL(sv_latent_prep_kernel<float>, dim3(a.T, 2), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(sv_latent_prep_kernel<uint16_t>, dim3(a.T, 2), dim3(256), 0, st, a);
+}
+void kr_sv_latent_q(const KrSvLatent& a, const float* q2, void* qn, float* qe, bool f32, hipStream_t st) {
+    if (a.T <= 0) return;
+    if (f32) hipLaunchKernelGGL(sv_latent_q_kernel<float>, dim3(a.T, a.heads), dim3(64), 0, st, a, q2, (float*)qn, qe);
+    else hipLaunchKernelGGL(sv_latent_q_kernel<uint16_t>, dim3(a.T, a.heads), dim3(64), 0, st, a, q2, (uint16_t*)qn, qe);
+}
+void kr_sv_head_rows(int T, int heads, int* seg, int* rows, int* group, hipStream_t st) {
+    const int n = T * heads > heads + 1 ? T * heads : heads + 1;
+    if (T <= 0) return;
+    hipLaunchKernelGGL(sv_head_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, st, T, heads, seg, rows, group);
 }
 
 void kr_sv_argmax(const float* logits, int R, int vocab, int* out, hipStream_t st) {

@@ -75,6 +75,12 @@ class ServeModelSpec:
     norm_eps: float
     layers: List[S.LayerSpec]
     tensors: Callable[["ServeModelSpec"], Iterator[Tuple[int, str, int, str]]]      # (layer, role, index, tensor name)
+    # how a layer is put together (`kr_serve_config` in include/krasis_hip.h); the defaults are one pre-normed block with mixer and feed-forward side by side
+    block_kind: int = S.BLOCK_PARALLEL
+    pre_norm: int = 1
+    post_norm: int = 0
+    norm_bias: Optional[int] = None      # None: layer norms carry a bias, RMS norms do not
+    residual_mult: float = 1.0
 
 
 _ARCHITECTURES: Dict[str, Callable[[dict], ServeModelSpec]] = {}
@@ -155,6 +161,78 @@ def lomutar_spec(cfg: dict) -> ServeModelSpec:
 
 
 register_architecture("Lomutar", lomutar_spec)
+
+
+# ---- Pamulix: x <- x + m * LN(mixer(x)), then x <- x + m * LN(ff(x)): the sublayers read the residual stream itself and a weight-only layer norm sits on
+# their OUTPUT.  Two mixers.  'attention': grouped key / value heads, RMS norm of q and k with a weight shared by the heads, no rotation; the score loses
+# slope_h * distance with slope_h = 2^(-8 (h + 1) / heads); a query sees the earlier keys of its own block of mask.size positions; the softmax denominator
+# carries an extra one; from the second layer marked v_mix on, the values are blended with the first such layer's values of the same token before they
+# are cached.  'latent_attention': queries and keys / values through normed low-rank latents, a rotated key part shared by the heads, by-parts scaled
+# rotation frequencies, plain causal softmax; the cache holds the latent and the shared part.  Feed-forward: SiLU-gated experts, the `top` largest of
+# (router logits + bias), softmax over the chosen logits.
+def _pamulix_tensors(spec: ServeModelSpec) -> Iterator[Tuple[int, str, int, str]]:
+    yield -1, "embed", 0, "embed"
+    yield -1, "final_norm_w", 0, "final.norm"
+    yield -1, "head", 0, "head"
+    for i, l in enumerate(spec.layers):
+        p = f"l{i}"
+        yield i, "post1_w", 0, f"{p}.norm1"
+        if l.mixer_kind == S.MIX_LATENT:
+            for r, n in (("dq", "dq"), ("dq_norm", "dq.norm"), ("uq", "uq"), ("dkv", "dkv"), ("dkv_norm", "dkv.norm"), ("uk", "uk"), ("uv", "uv")):
+                yield i, r, 0, f"{p}.mix.{n}"
+        else:
+            for r, n in (("q", "q"), ("k", "k"), ("v", "v"), ("q_norm", "q.norm"), ("k_norm", "k.norm")):
+                yield i, r, 0, f"{p}.mix.{n}"
+            if l.v_mix == S.VMIX_BLEND:
+                yield i, "vmix", 0, f"{p}.mix.vmix"
+        yield i, "o", 0, f"{p}.mix.o"
+        if l.mlp_kind == S.MLP_MOE:
+            yield i, "post2_w", 0, f"{p}.norm2"
+            yield i, "router", 0, f"{p}.mlp.router"
+            yield i, "router_bias", 0, f"{p}.mlp.router.b"
+            for e in range(l.experts):
+                for r in ("gate", "up", "down"):
+                    yield i, f"expert_{r}", e, f"{p}.mlp.e{e}.{r}"
+
+
+def pamulix_spec(cfg: dict) -> ServeModelSpec:
+    layers: List[S.LayerSpec] = []
+    mixing_seen = False
+    for i, lc in enumerate(cfg["layers"]):
+        kind, m = lc.get("type"), lc["mixer"]
+        if kind == "attention":
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                            qk_unit_norm=S.QKNORM_WEIGHTED, scale=float(m["scale"]), chunk=int((m.get("mask") or {}).get("size", 0)), has_sink=S.SINK_ZERO,
+                            dist_bias=1, dist_bias_exp=8.0)
+            if m.get("v_mix"):
+                l.v_mix = S.VMIX_BLEND if mixing_seen else S.VMIX_FIRST
+                mixing_seen = True
+        elif kind == "latent_attention":
+            rot = m["rot"]
+            if int(rot["dims"]) != int(m["rot_dim"]):
+                raise ValueError(f"layer {i}: the rotated part has {m['rot_dim']} coordinates, the rotation {rot['dims']}")
+            l = S.LayerSpec(heads=int(m["heads"]), kv_heads=1, dim=int(m["dim"]), vdim=int(m["vdim"]), mixer_kind=S.MIX_LATENT, q_rank=int(m["q_rank"]),
+                            kv_rank=int(m["kv_rank"]), rot_dims=int(m["rot_dim"]), rot_interleaved=1, rot_base=float(rot["base"]), scale=float(m["scale"]))
+            sc = rot.get("scaling")
+            if sc:
+                l.rot_scaling, l.rot_factor = S.ROT_BY_PARTS, float(sc["factor"])
+                l.rot_original, l.rot_fast, l.rot_slow = float(sc["original"]), float(sc["fast"]), float(sc["slow"])
+        else:
+            raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
+        mlp = lc.get("mlp")
+        if mlp is not None:
+            if mlp.get("kind") != "moe":
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r}")
+            r, ex = mlp["router"], mlp["expert"]
+            l.mlp_kind, l.experts, l.top, l.groups, l.keep = S.MLP_MOE, int(r["experts"]), int(r["top"]), 1, 1
+            l.renorm, l.router_bias = 1, 1      # the softmax over all logits, renormalised over the chosen ones, is the softmax over the chosen ones
+            l.expert_ff, l.expert_act = int(ex["ff"]), S.ACT_SILU
+        layers.append(l)
+    return ServeModelSpec(vocab=int(cfg["vocab"]), width=int(cfg["width"]), norm_kind=S.NORM_LAYER, norm_eps=float(cfg["norm"]["eps"]), layers=layers,
+                          tensors=_pamulix_tensors, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=0, post_norm=1, norm_bias=0, residual_mult=float(cfg["residual_mult"]))
+
+
+register_architecture("Pamulix", pamulix_spec)
 
 
 def read_config(model_dir: str) -> dict:

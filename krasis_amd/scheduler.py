@@ -23,7 +23,8 @@ class BatchEngine:
             raise ValueError(f"dtype {dtype!r}: bfloat16 | float32")
         self.spec = spec
         self.store = S.ServeStore(spec.vocab, spec.width, spec.layers, dtype=_DTYPES[dtype], norm_kind=spec.norm_kind, norm_eps=spec.norm_eps,
-                                  max_slots=max_slots, pool_tokens=max_tokens, device=device, build=build)
+                                  max_slots=max_slots, pool_tokens=max_tokens, device=device, build=build, block_kind=spec.block_kind, pre_norm=spec.pre_norm,
+                                  post_norm=spec.post_norm, norm_bias=spec.norm_bias, residual_mult=spec.residual_mult)
         self.vocab = spec.vocab
         self._slot: Dict[object, int] = {}
 

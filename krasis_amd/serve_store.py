@@ -16,14 +16,23 @@ BF16, F32 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
 MLP_NONE, MLP_DENSE, MLP_MOE = 0, 1, 2
 ACT_GELU_TANH, ACT_CLAMPED_SWIGLU, ACT_SILU = 0, 1, 2
+BLOCK_PARALLEL, BLOCK_SEQUENTIAL = 0, 1
+MIX_ATTENTION, MIX_LATENT = 0, 1
+QKNORM_NONE, QKNORM_AFTER_ROT, QKNORM_WEIGHTED = 0, 1, 2
+SINK_NONE, SINK_TENSOR, SINK_ZERO = 0, 1, 2
+ROT_LINEAR, ROT_BY_PARTS = 0, 1
+VMIX_NONE, VMIX_FIRST, VMIX_BLEND = 0, 1, 2
 PAGE_TOKENS = 64
 ROLES = {n: i for i, n in enumerate(["embed", "final_norm_w", "final_norm_b", "head", "norm_w", "norm_b", "q", "k", "v", "o", "sink", "gate", "up", "down",
-                                     "router", "expert_gate", "expert_up", "expert_down", "shared_gate", "shared_up", "shared_down"])}
+                                     "router", "expert_gate", "expert_up", "expert_down", "shared_gate", "shared_up", "shared_down",
+                                     "norm2_w", "norm2_b", "post1_w", "post1_b", "post2_w", "post2_b", "q_norm", "k_norm", "vmix", "router_bias",
+                                     "dq", "dq_norm", "uq", "dkv", "dkv_norm", "uk", "uv"])}
 
 
 @dataclass
 class LayerSpec:
-    """One layer: attention mixer + parallel feed-forward on one normed input (field meanings: `kr_serve_layer` in include/krasis_hip.h)."""
+    """One layer: a mixer (attention, or attention through latents) and a feed-forward, beside or after one another (field meanings: `kr_serve_layer`
+    in include/krasis_hip.h)."""
     heads: int
     kv_heads: int
     dim: int
@@ -51,17 +60,33 @@ class LayerSpec:
     expert_alpha: float = 1.702
     shared_ff: int = 0
     shared_limit: float = 0.0
+    mixer_kind: int = MIX_ATTENTION
+    q_rank: int = 0
+    kv_rank: int = 0
+    rot_scaling: int = ROT_LINEAR
+    rot_original: float = 0.0
+    rot_fast: float = 0.0
+    rot_slow: float = 0.0
+    chunk: int = 0
+    dist_bias: int = 0
+    dist_bias_exp: float = 8.0
+    v_mix: int = VMIX_NONE
+    router_bias: int = 0
 
 
 class ServeStore:
     def __init__(self, vocab: int, width: int, layers: Sequence[LayerSpec], dtype: int = BF16, norm_kind: int = NORM_LAYER, norm_eps: float = 1e-5,
-                 max_slots: int = 4, pool_tokens: int = 4096, page_tokens: int = PAGE_TOKENS, device: int = 0, build: bool = False):
+                 max_slots: int = 4, pool_tokens: int = 4096, page_tokens: int = PAGE_TOKENS, device: int = 0, build: bool = False,
+                 block_kind: int = BLOCK_PARALLEL, pre_norm: int = 1, post_norm: int = 0, norm_bias: Optional[int] = None, residual_mult: float = 1.0):
         self._lib = load_serve_library(build=build)
         self.vocab, self.width, self.layers, self.dtype = vocab, width, list(layers), dtype
         self.page_tokens = page_tokens
         pool_tokens = (max(pool_tokens, page_tokens) + page_tokens - 1) // page_tokens * page_tokens
         self.pool_tokens, self.max_slots = pool_tokens, max_slots
-        cfg = ServeConfigC(vocab, width, len(self.layers), dtype, norm_kind, norm_eps, max_slots, page_tokens, pool_tokens)
+        if norm_bias is None:
+            norm_bias = int(norm_kind == NORM_LAYER)
+        cfg = ServeConfigC(vocab, width, len(self.layers), dtype, norm_kind, norm_eps, max_slots, page_tokens, pool_tokens, block_kind, pre_norm, post_norm, norm_bias,
+                           residual_mult)
         arr = (ServeLayerC * len(self.layers))()
         for i, l in enumerate(self.layers):
             for f in fields(LayerSpec):
@@ -90,7 +115,7 @@ class ServeStore:
             src = F32
         else:
             raise ValueError(f"tensor dtype {a.dtype}: bf16 bit patterns (uint16) or float32")
-        rows, cols = (1, a.size) if a.ndim == 1 else a.shape
+        rows, cols = (1, a.size) if a.ndim <= 1 else a.shape
         check_serve(self._lib.kr_serve_set_tensor(self._h, layer, ROLES[role], index, a.ctypes.data, src, rows, cols))
 
     def fill_synthetic(self, seed: int = 1, amp: float = 1.0) -> None:
