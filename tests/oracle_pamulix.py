@@ -127,7 +127,8 @@ def chunked_bias_attention(q, k, v, scale, chunk):
 
 
 def mix_values(v, v_first, lam):
-    return (1.0 - lam) * v + lam * v_first
+    """per token, over all value heads laid end to end"""
+    return (1.0 - lam) * v + lam * v_first.reshape(v.shape)
 
 
 def grouped_attention(h, W, p, m, eps, first_values):
