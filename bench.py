@@ -347,6 +347,9 @@ def parse():
                          "sizes -- prompt pass and decode throughput, kernel-family times -- beside the closest model of the decode graph (GQA + softmax top-k MoE, INT4) at "
                          "the same sizes; prints its own JSON line")
     ap.add_argument("--arch-sizes", default="small,large", help="sizes of --arch-compare (ARCH_SIZES)")
+    ap.add_argument("--arch-design", default="lomutar", choices=["lomutar", "pamulix"],
+                    help="which layer-described design --arch-compare measures: lomutar (beside the decode graph's GQA + MoE model) or pamulix (beside Lomutar, "
+                         "both on the batched serving store, at the same layer sizes)")
     return ap.parse_args()
 
 
@@ -450,6 +453,129 @@ def arch_compare(args):
             res["gqa_moe_error"] = repr(ex)
         finally:
             Q235 = saved
+        out["sizes"][name] = res
+    flush_native_stdout()
+    print(json.dumps(out), flush=True)
+    return out
+
+
+SERVE_FAMILIES = ["norm", "gemm", "qk_prep+rope", "attention", "router+sort", "activation", "residual", "embed+argmax"]
+F32_MATRIX_PEAK_TFLOPS = 157.3      # v_mfma_f32_16x16x4_f32: 256 flops per CU and cycle x 256 CUs x 2.4 GHz
+
+
+def serve_measure(eng, V, P, rng, decode_batches=(1, 4)):
+    """Prompt pass of P tokens (median of three, then one pass with kernel-family times) and decode steps at position ~ P for 1 and 4 requests on a batched
+    serving engine with random weights.  Returns raw times; the caller prices them against its own flop / byte counts."""
+    import numpy as np
+    toks = lambda n: [int(x) for x in rng.integers(0, V, n)]
+
+    def prompt_pass(profile=False):
+        eng.store.set_profiling(profile)
+        t0 = time.perf_counter(); eng.step([("p", toks(P), [P - 1])], logits=False); dt = time.perf_counter() - t0
+        fam = eng.store.profile() if profile else None
+        eng.store.set_profiling(False)
+        eng.finish("p")
+        return dt, fam
+    prompt_pass()
+    dt = sorted(prompt_pass()[0] for _ in range(3))[1]
+    _, fam = prompt_pass(profile=True)
+    out = {"prefill_s": dt, "prefill_family_ms": list(fam), "decode": {}}
+    for B in decode_batches:
+        for b in range(B):
+            eng.step([(("d", b), toks(P), [])], logits=False)
+        ent = lambda: [(("d", b), toks(1), [0]) for b in range(B)]
+        for _ in range(20):
+            eng.step(ent(), logits=False)
+        n = 50
+        t0 = time.perf_counter()
+        for _ in range(n):
+            eng.step(ent(), logits=False)
+        dts = (time.perf_counter() - t0) / n
+        eng.store.set_profiling(True)
+        for _ in range(10):
+            eng.step(ent(), logits=False)
+        famd = [v / 10 for v in eng.store.profile()]; eng.store.set_profiling(False)
+        out["decode"][B] = {"s_per_step": dts, "family_ms": famd}
+        for b in range(B):
+            eng.finish(("d", b))
+    return out
+
+
+def arch_compare_pamulix(args):
+    """The Pamulix design beside Lomutar, both on the batched serving store with random bf16 weights, at the layer sizes of ARCH_SIZES.  Pamulix layers:
+    chunked attention with a distance bias (the size's heads / window as its chunk) and attention through latents (kv_rank 512 + 64 rotated, query rank
+    width * 3 / 8, heads of 128 + 64), SiLU experts behind a top-k router, no shared expert; order attention, latent, attention, attention, ...  Three
+    Pamulix models per size: the mixed order (the throughput), and one mixer kind alone each (what its attention kernel reaches)."""
+    import numpy as np
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    out = {"metric": "arch_compare_pamulix_vs_lomutar", "unit": "tok/s", "sizes": {}}
+    for name in [x for x in args.arch_sizes.split(",") if x]:
+        z = ARCH_SIZES[name]; W, H, G, D, E, k, F, L, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "experts", "top", "ff", "layers", "vocab", "prompt"))
+        Rk, Rr, Qr = 512, 64, W * 3 // 8
+        res = {"shape": dict(z, kv_rank=Rk, rot_dim=Rr, q_rank=Qr)}
+
+        def attention_layer(first):
+            return S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, chunk=z["window"], has_sink=S.SINK_ZERO, dist_bias=1,
+                               v_mix=S.VMIX_FIRST if first else S.VMIX_BLEND, mlp_kind=S.MLP_MOE, experts=E, top=k, groups=1, keep=1, renorm=1, router_bias=1, expert_ff=F,
+                               expert_act=S.ACT_SILU)
+
+        def latent_layer():
+            return S.LayerSpec(heads=H, kv_heads=1, dim=D, vdim=D, mixer_kind=S.MIX_LATENT, q_rank=Qr, kv_rank=Rk, rot_dims=Rr, rot_base=1e4, rot_factor=40.0,
+                               rot_scaling=S.ROT_BY_PARTS, rot_original=4096.0, rot_fast=32.0, rot_slow=1.0, scale=(D + Rr) ** -0.5, mlp_kind=S.MLP_MOE, experts=E, top=k,
+                               groups=1, keep=1, renorm=1, router_bias=1, expert_ff=F, expert_act=S.ACT_SILU)
+
+        def pamulix(kinds):
+            layers, seen = [], False
+            for kd in kinds:
+                layers.append(latent_layer() if kd == "L" else attention_layer(not seen))
+                seen = seen or kd == "A"
+            spec = R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=0, post_norm=1, norm_bias=0, residual_mult=0.5)
+            eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+            eng.load_synthetic(seed=7, amp=1.0)
+            return eng
+        w_moe_tok = k * 3 * W * F
+        w_att = (H * D + 2 * G * D) * W + W * H * D
+        w_lat = (Qr + Rk + Rr) * W + H * (D + Rr) * Qr + H * D * Rk * 2 + W * H * D
+        att_flops = 2.0 * 2 * H * D * sum(min(i % z["window"] + 1, z["window"]) for i in range(P))            # per attention layer and prompt
+        lat_flops = 2.0 * H * (2 * Rk + Rr) * sum(i + 1 for i in range(P))                                   # per latent layer: keys 576 wide, values 512
+        order = "".join("L" if i == 1 else "A" for i in range(L))
+        for label, kinds in (("mixed_" + order, order), ("attention_only", "A" * L), ("latent_only", "L" * L)):
+            eng = pamulix(kinds)
+            m = serve_measure(eng, V, P, np.random.default_rng(3), decode_batches=(1, 4) if label.startswith("mixed") else (1,))
+            nA, nL = kinds.count("A"), kinds.count("L")
+            macs_tok = nA * w_att + nL * w_lat + L * (w_moe_tok + E * W)
+            fam = m["prefill_family_ms"]
+            r = {"prefill": {"tok_s": P / m["prefill_s"], "ms": m["prefill_s"] * 1e3, "tokens": P, "family_ms": {n: round(v, 3) for n, v in zip(SERVE_FAMILIES, fam)},
+                             "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                             "attention_family_TFLOPs": (nA * att_flops + nL * lat_flops) / (fam[3] * 1e-3) / 1e12}}
+            r["prefill"]["attention_frac_of_f32_matrix_peak"] = r["prefill"]["attention_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
+            for B, d in m["decode"].items():
+                byts = 2.0 * (nA * w_att + nL * w_lat + L * (min(E, B * k) * 3 * W * F + E * W) + V * W)
+                r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_bytes_per_step": byts,
+                                       "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
+                                       "gemm_family_frac_of_hbm_peak": byts / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            res["pamulix_" + label] = r
+            del eng; gc.collect()
+        # ---------------- Lomutar at the same sizes (windowed attention with a sink, rotation, group-limited router, clamped experts + shared expert)
+        layers = [S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, rot_dims=D // 2, rot_base=1e6, rot_factor=2.0, qk_unit_norm=1, scale=D ** -0.5, window=z["window"], has_sink=1,
+                              mlp_kind=S.MLP_MOE, experts=E, top=k, groups=4, keep=2, expert_ff=F, expert_limit=7.0, shared_ff=F, shared_limit=7.0) for _ in range(L)]
+        eng = SCH.BatchEngine(R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None), dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+        eng.load_synthetic(seed=7, amp=1.0)
+        m = serve_measure(eng, V, P, np.random.default_rng(3))
+        macs_tok = L * (w_att + (k + 1) * 3 * W * F + E * W)
+        fam = m["prefill_family_ms"]
+        lo_flops = L * 2.0 * 2 * H * D * sum(min(i + 1, z["window"]) for i in range(P))
+        r = {"prefill": {"tok_s": P / m["prefill_s"], "ms": m["prefill_s"] * 1e3, "tokens": P, "family_ms": {n: round(v, 3) for n, v in zip(SERVE_FAMILIES, fam)},
+                         "gemm_family_frac_of_bf16_peak": 2.0 * P * (macs_tok + V * W / P) / (fam[1] * 1e-3) / 1e12 / F16_PEAK_TFLOPS,
+                         "attention_family_TFLOPs": lo_flops / (fam[3] * 1e-3) / 1e12}}
+        r["prefill"]["attention_frac_of_f32_matrix_peak"] = r["prefill"]["attention_family_TFLOPs"] / F32_MATRIX_PEAK_TFLOPS
+        for B, d in m["decode"].items():
+            byts = 2.0 * (L * (w_att + (min(E, B * k) + 1) * 3 * W * F + E * W * 2) + V * W)
+            r["decode_b%d" % B] = {"tok_s": B / d["s_per_step"], "ms_per_step": d["s_per_step"] * 1e3, "weight_bytes_per_step": byts,
+                                   "frac_of_hbm_peak": byts / d["s_per_step"] / 1e9 / HBM_PEAK_GBS, "family_ms": {n: round(v, 4) for n, v in zip(SERVE_FAMILIES, d["family_ms"])},
+                                   "gemm_family_frac_of_hbm_peak": byts / (d["family_ms"][1] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        res["lomutar"] = r
+        del eng; gc.collect()
         out["sizes"][name] = res
     flush_native_stdout()
     print(json.dumps(out), flush=True)
@@ -1414,7 +1540,7 @@ def main_multi(args, torch, dist, world, rank, local_rank):
 def main():
     args = parse()
     if args.arch_compare:
-        return arch_compare(args)
+        return arch_compare_pamulix(args) if args.arch_design == "pamulix" else arch_compare(args)
     import torch
     import torch.distributed as dist
 

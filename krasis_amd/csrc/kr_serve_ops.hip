@@ -438,22 +438,28 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
 #pragma unroll
             for (int kb = 0; kb < 4; kb++) {
                 const T* k = kp + (size_t)prow[kb] * a.ldk + (size_t)g * dim + qd * DQ;
-                sv_u4 kv[DQ / VEC];
-#pragma unroll
-                for (int u = 0; u < DQ / VEC; u++) kv[u] = *reinterpret_cast<const sv_u4*>(k + u * VEC);
+                // a key row's quarter in batches of at most PB 16-byte pieces: long rows (a latent cache row) must not hold all of it in registers at once
+                constexpr int NP = DQ / VEC, PB = NP <= 8 ? NP : 6;
                 sv_f4 c = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int u = 0; u < DQ / VEC; u++) {
-                    float kf[VEC];
-                    if constexpr (sizeof(T) == 2) {
+                for (int u0 = 0; u0 < NP; u0 += PB) {
+                    sv_u4 kv[PB];
 #pragma unroll
-                        for (int i = 0; i < 4; i++) { kf[2 * i] = __uint_as_float(kv[u][i] << 16); kf[2 * i + 1] = __uint_as_float(kv[u][i] & 0xFFFF0000u); }
-                    } else {
+                    for (int u = 0; u < PB; u++) if (u0 + u < NP) kv[u] = *reinterpret_cast<const sv_u4*>(k + (u0 + u) * VEC);
 #pragma unroll
-                        for (int i = 0; i < 4; i++) kf[i] = __uint_as_float(kv[u][i]);
+                    for (int u = 0; u < PB; u++) {
+                        if (u0 + u >= NP) continue;
+                        float kf[VEC];
+                        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) { kf[2 * i] = __uint_as_float(kv[u][i] << 16); kf[2 * i + 1] = __uint_as_float(kv[u][i] & 0xFFFF0000u); }
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) kf[i] = __uint_as_float(kv[u][i]);
+                        }
+#pragma unroll
+                        for (int i = 0; i < VEC; i++) c = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], q[(u0 + u) * VEC + i], c, 0, 0, 0);
                     }
-#pragma unroll
-                    for (int i = 0; i < VEC; i++) c = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[i], q[u * VEC + i], c, 0, 0, 0);
                 }
                 st[kb] = c;
             }
@@ -481,34 +487,41 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
 #pragma unroll
             for (int d = 0; d < DB; d++) acc[d] *= alpha;
             // ---- O^T += V^T P^T: key (kb, 4 qd + i) -> this lane reads its DB value columns of that key's row
+            // wide values (DB > 16) go through in column batches of DC, so that one batch of four keys' values is in registers at a time
+            constexpr int DC = DB <= 16 ? DB : 8;
 #pragma unroll
             for (int kb = 0; kb < 4; kb++) {
-                float vf[4][DB];
+                int prk[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int pr = __shfl(prow[kb], 4 * qd + i);
-                    const T* vr = vp + (size_t)pr * a.ldv + (size_t)g * vdim + row * DB;
-                    if constexpr ((DB * sizeof(T)) % 16 == 0) {
+                for (int i = 0; i < 4; i++) prk[i] = __shfl(prow[kb], 4 * qd + i);
 #pragma unroll
-                        for (int u = 0; u < DB / VEC; u++) {
-                            const sv_u4 vv = *reinterpret_cast<const sv_u4*>(vr + u * VEC);
-                            if constexpr (sizeof(T) == 2) {
+                for (int d0 = 0; d0 < DB; d0 += DC) {
+                    float vf[4][DC];
 #pragma unroll
-                                for (int e = 0; e < 4; e++) { vf[i][u * VEC + 2 * e] = __uint_as_float(vv[e] << 16); vf[i][u * VEC + 2 * e + 1] = __uint_as_float(vv[e] & 0xFFFF0000u); }
-                            } else {
+                    for (int i = 0; i < 4; i++) {
+                        const T* vr = vp + (size_t)prk[i] * a.ldv + (size_t)g * vdim + row * DB + d0;
+                        if constexpr ((DC * sizeof(T)) % 16 == 0 && (DB * sizeof(T)) % 16 == 0) {
 #pragma unroll
-                                for (int e = 0; e < 4; e++) vf[i][u * VEC + e] = __uint_as_float(vv[e]);
+                            for (int u = 0; u < DC / VEC; u++) {
+                                const sv_u4 vv = *reinterpret_cast<const sv_u4*>(vr + u * VEC);
+                                if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) { vf[i][u * VEC + 2 * e] = __uint_as_float(vv[e] << 16); vf[i][u * VEC + 2 * e + 1] = __uint_as_float(vv[e] & 0xFFFF0000u); }
+                                } else {
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) vf[i][u * VEC + e] = __uint_as_float(vv[e]);
+                                }
                             }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < DC; e++) vf[i][e] = sv_ld(vr + e);
                         }
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < DB; e++) vf[i][e] = sv_ld(vr + e);
                     }
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+#pragma unroll
+                        for (int d = 0; d < DC; d++) acc[d0 + d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][d], st[kb][i], acc[d0 + d], 0, 0, 0);
                 }
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int d = 0; d < DB; d++) acc[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[i][d], st[kb][i], acc[d], 0, 0, 0);
             }
         }
         // ---- the four waves' states -> one, in wave order; an unsplit launch adds the sink and writes the output, a split one leaves (maximum, denominator, sums)
@@ -924,6 +937,10 @@ static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
     if (dq == 8 && db == 16) SV_MF(8, 16);
     if (dq == 8 && db == 1) SV_MF(8, 1);
     if (dq == 16 && db == 1) SV_MF(16, 1);
+    // latent cache rows: [latent | rotated part] as the key, the latent as the value (512 + 64, 256 + 64, 128 + 64, 64 + 64 and the like)
+    if (dq == 144 && db == 32) SV_MF(144, 32);
+    if (dq == 80 && db == 16) SV_MF(80, 16);
+    if (dq == 48 && db == 8) SV_MF(48, 8);
 #undef SV_MF
     return false;
 }

