@@ -501,6 +501,32 @@ def serve_measure(eng, V, P, rng, decode_batches=(1, 4)):
     return out
 
 
+def pamulix_serve_engine(z, kinds, kv_rank=512, rot_dim=64):
+    """A Pamulix model with random bf16 weights on the batched serving store at the layer sizes z (ARCH_SIZES); kinds: one letter per layer, A = chunked
+    attention with a distance bias, L = attention through latents"""
+    from krasis_amd import model_registry as R, scheduler as SCH, serve_store as S
+    W, H, G, D, E, k, F, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "experts", "top", "ff", "vocab", "prompt"))
+    Rk, Rr, Qr = kv_rank, rot_dim, W * 3 // 8
+
+    def attention_layer(first):
+        return S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, chunk=z["window"], has_sink=S.SINK_ZERO, dist_bias=1,
+                           v_mix=S.VMIX_FIRST if first else S.VMIX_BLEND, mlp_kind=S.MLP_MOE, experts=E, top=k, groups=1, keep=1, renorm=1, router_bias=1, expert_ff=F,
+                           expert_act=S.ACT_SILU)
+
+    def latent_layer():
+        return S.LayerSpec(heads=H, kv_heads=1, dim=D, vdim=D, mixer_kind=S.MIX_LATENT, q_rank=Qr, kv_rank=Rk, rot_dims=Rr, rot_base=1e4, rot_factor=40.0,
+                           rot_scaling=S.ROT_BY_PARTS, rot_original=4096.0, rot_fast=32.0, rot_slow=1.0, scale=(D + Rr) ** -0.5, mlp_kind=S.MLP_MOE, experts=E, top=k,
+                           groups=1, keep=1, renorm=1, router_bias=1, expert_ff=F, expert_act=S.ACT_SILU)
+    layers, seen = [], False
+    for kd in kinds:
+        layers.append(latent_layer() if kd == "L" else attention_layer(not seen))
+        seen = seen or kd == "A"
+    spec = R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=0, post_norm=1, norm_bias=0, residual_mult=0.5)
+    eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+    eng.load_synthetic(seed=7, amp=1.0)
+    return eng
+
+
 def arch_compare_pamulix(args):
     """The Pamulix design beside Lomutar, both on the batched serving store with random bf16 weights, at the layer sizes of ARCH_SIZES.  Pamulix layers:
     chunked attention with a distance bias (the size's heads / window as its chunk) and attention through latents (kv_rank 512 + 64 rotated, query rank
@@ -514,25 +540,7 @@ def arch_compare_pamulix(args):
         Rk, Rr, Qr = 512, 64, W * 3 // 8
         res = {"shape": dict(z, kv_rank=Rk, rot_dim=Rr, q_rank=Qr)}
 
-        def attention_layer(first):
-            return S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, qk_unit_norm=S.QKNORM_WEIGHTED, scale=D ** -0.5, chunk=z["window"], has_sink=S.SINK_ZERO, dist_bias=1,
-                               v_mix=S.VMIX_FIRST if first else S.VMIX_BLEND, mlp_kind=S.MLP_MOE, experts=E, top=k, groups=1, keep=1, renorm=1, router_bias=1, expert_ff=F,
-                               expert_act=S.ACT_SILU)
-
-        def latent_layer():
-            return S.LayerSpec(heads=H, kv_heads=1, dim=D, vdim=D, mixer_kind=S.MIX_LATENT, q_rank=Qr, kv_rank=Rk, rot_dims=Rr, rot_base=1e4, rot_factor=40.0,
-                               rot_scaling=S.ROT_BY_PARTS, rot_original=4096.0, rot_fast=32.0, rot_slow=1.0, scale=(D + Rr) ** -0.5, mlp_kind=S.MLP_MOE, experts=E, top=k,
-                               groups=1, keep=1, renorm=1, router_bias=1, expert_ff=F, expert_act=S.ACT_SILU)
-
-        def pamulix(kinds):
-            layers, seen = [], False
-            for kd in kinds:
-                layers.append(latent_layer() if kd == "L" else attention_layer(not seen))
-                seen = seen or kd == "A"
-            spec = R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None, block_kind=S.BLOCK_SEQUENTIAL, pre_norm=0, post_norm=1, norm_bias=0, residual_mult=0.5)
-            eng = SCH.BatchEngine(spec, dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
-            eng.load_synthetic(seed=7, amp=1.0)
-            return eng
+        pamulix = lambda kinds: pamulix_serve_engine(z, kinds)  # noqa: E731
         w_moe_tok = k * 3 * W * F
         w_att = (H * D + 2 * G * D) * W + W * H * D
         w_lat = (Qr + Rk + Rr) * W + H * (D + Rr) * Qr + H * D * Rk * 2 + W * H * D

@@ -1,6 +1,7 @@
-"""Probe: the Lomutar design on the batched serving store at one of bench.py's --arch-compare sizes, random bf16 weights.
-    python tools/probes/serve_profile.py <small|large> prefill      three prompt passes of the size's prompt length
-    python tools/probes/serve_profile.py <small|large> decode       decode steps of 1 and of 4 requests at the end of such a prompt, graphs on / off
+"""Probe: a layer-described design on the batched serving store at one of bench.py's --arch-compare sizes, random bf16 weights.
+    python tools/probes/serve_profile.py <small|large> prefill [design]     three prompt passes of the size's prompt length
+    python tools/probes/serve_profile.py <small|large> decode [design]      decode steps of 1 and of 4 requests at the end of such a prompt, graphs on / off
+design: lomutar (default), or pamulix:<one letter per layer, A = chunked attention, L = attention through latents>, e.g. pamulix:ALAA
 Run under `rocprofv3 --kernel-trace --stats` for the kernel tables in profiles/serve_*."""
 import os
 import sys
@@ -16,10 +17,14 @@ name = sys.argv[1] if len(sys.argv) > 1 else "small"
 mode = sys.argv[2] if len(sys.argv) > 2 else "decode"
 z = bench.ARCH_SIZES[name]
 W, H, G, D, E, k, F, L, V, P = (z[c] for c in ("width", "heads", "kv_heads", "dim", "experts", "top", "ff", "layers", "vocab", "prompt"))
+design = sys.argv[3] if len(sys.argv) > 3 else "lomutar"
 layers = [S.LayerSpec(heads=H, kv_heads=G, dim=D, vdim=D, rot_dims=D // 2, rot_base=1e6, rot_factor=2.0, qk_unit_norm=1, scale=D ** -0.5, window=z["window"], has_sink=1,
                       mlp_kind=S.MLP_MOE, experts=E, top=k, groups=4, keep=2, expert_ff=F, expert_limit=7.0, shared_ff=F, shared_limit=7.0) for _ in range(L)]
-eng = SCH.BatchEngine(R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None), dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
-eng.load_synthetic(seed=7, amp=1.0)
+if design.startswith("pamulix:"):
+    eng = bench.pamulix_serve_engine(z, design.split(":", 1)[1])
+else:
+    eng = SCH.BatchEngine(R.ServeModelSpec(V, W, S.NORM_LAYER, 1e-5, layers, None), dtype="bfloat16", max_tokens=4 * (P + 256), max_slots=4)
+    eng.load_synthetic(seed=7, amp=1.0)
 rng = np.random.default_rng(3)
 toks = lambda n: [int(x) for x in rng.integers(0, V, n)]  # noqa: E731
 if mode == "prefill":
