@@ -67,15 +67,15 @@ def test_registry_and_checkpoint_roundtrip(tmp_path):
 
 def test_oracle_rotation_table():
     """by-parts scaling: pairs below the ramp keep base^(-2i/dims), pairs above it are divided by the factor, cos and sin are stretched"""
-    f, mult = O.yarn_table(32, 10000.0, 4.0, 2048, 32.0, 1.0)
+    f, mult = O.yarn_table(32, 10000.0, 6.0, 1024, 16.0, 2.0)
     plain, one = O.plain_table(32, 10000.0)
-    assert one == 1.0 and abs(mult - (0.1 * math.log(4.0) + 1.0)) < 1e-15
-    lo = math.floor(32 * math.log(2048 / (2 * math.pi * 32.0)) / (2 * math.log(10000.0)))
-    hi = math.ceil(32 * math.log(2048 / (2 * math.pi * 1.0)) / (2 * math.log(10000.0)))
+    assert one == 1.0 and abs(mult - (0.1 * math.log(6.0) + 1.0)) < 1e-15
+    lo = math.floor(32 * math.log(1024 / (2 * math.pi * 16.0)) / (2 * math.log(10000.0)))
+    hi = math.ceil(32 * math.log(1024 / (2 * math.pi * 2.0)) / (2 * math.log(10000.0)))
     assert 0 < lo < hi < 16
-    assert np.allclose(f[:lo + 1], plain[:lo + 1]) and np.allclose(f[hi:], plain[hi:] / 4.0)
+    assert np.allclose(f[:lo + 1], plain[:lo + 1]) and np.allclose(f[hi:], plain[hi:] / 6.0)
     mid = (lo + hi) // 2
-    assert plain[mid] / 4.0 < f[mid] < plain[mid]
+    assert plain[mid] / 6.0 < f[mid] < plain[mid]
     x = np.random.default_rng(0).standard_normal((5, 2, 40))
     y = O.rotate_pairs(x, np.arange(5), f, mult)
     assert np.array_equal(y[:, :, 32:], x[:, :, 32:]) and np.allclose(y[0, :, :32], x[0, :, :32] * mult)     # the tail passes; position 0 only stretches

@@ -386,6 +386,21 @@ def test_long_decoding_through_pages_and_chunks():
     assert rel(np.stack(rows), ref[20:]) < 2e-4
 
 
+@pytest.mark.parametrize("mixer", [O.latent(16, 8, 64, 8, 16, 512, base=1e4, scaling=(8.0, 64, 8.0, 1.0), scale=0.2), O.latent(4, 24, 64, 8, 16, 256, base=1e4, scale=0.15),
+                                   O.latent(2, 8, 64, 24, 16, 128, base=1e3, scale=0.2), O.attn(8, 2, 64, 64, 0, scale=0.12)])
+def test_decoding_over_a_long_cache_on_the_matrix_path(mixer):
+    """decode steps whose keys are split over several workgroups (partial states merged by a second launch), for the long cache rows of latent layers"""
+    cfg = small_model([O.layer(mixer, O.moe(4, 2, 16))]); W = O.random_weights(cfg, 45); n = 600; toks = tokens(cfg, n, 46)
+    ref, _ = O.forward(cfg, W, toks)
+    eng = engine(cfg, W)
+    eng.step([("a", toks[:570], [])])
+    rows = []
+    for p in range(570, n):
+        lg, _ = eng.step([("a", [toks[p]], [0])])
+        rows.append(lg[0])
+    assert rel(np.stack(rows), ref[570:]) < 2e-4
+
+
 def greedy_oracle(cfg, W, prompt, n_new):
     seq, out, margins = list(prompt), [], []
     for _ in range(n_new):
