@@ -568,20 +568,30 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
     }
 }
 
-// the partial states of a split launch -> output: one wave per (token, head)
+// the partial states of a split launch -> output: one workgroup per (token, head).  The splits' weights exp(m_s - M) are formed once (LDS); a thread then owns
+// value columns and its loads over the splits do not depend on one another
 template <typename T>
-__global__ void __launch_bounds__(64) sv_attn_merge_kernel(const KrSvAttn a) {
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ void __launch_bounds__(256) sv_attn_merge_kernel(const KrSvAttn a) {
+    extern __shared__ float wsp[];           // [nsplit] weight of every split, then 1 / denominator
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const size_t base = ((size_t)t * a.heads + h) * a.nsplit;
     float M = a.sink ? a.sink[h] : -INFINITY;
     for (int s = 0; s < a.nsplit; s++) M = fmaxf(M, a.part_ml[(base + s) * 2]);
-    float L = a.sink ? expf(a.sink[h] - M) : 0.0f;
-    for (int s = 0; s < a.nsplit; s++) { const float ms = a.part_ml[(base + s) * 2]; if (ms != -INFINITY) L += a.part_ml[(base + s) * 2 + 1] * expf(ms - M); }
+    for (int s = tid; s < a.nsplit; s += 256) { const float ms = a.part_ml[(base + s) * 2]; wsp[s] = ms == -INFINITY ? 0.0f : expf(ms - M); }
+    __syncthreads();
+    if (tid == 0) {
+        float L = a.sink ? expf(a.sink[h] - M) : 0.0f;
+        for (int s = 0; s < a.nsplit; s++) if (wsp[s] != 0.0f) L = __builtin_fmaf(a.part_ml[(base + s) * 2 + 1], wsp[s], L);
+        wsp[a.nsplit] = 1.0f / L;
+    }
+    __syncthreads();
+    const float inv = wsp[a.nsplit];
     T* o = (T*)a.out + ((size_t)t * a.heads + h) * a.vdim;
-    for (int d = lane; d < a.vdim; d += 64) {
+    for (int d = tid; d < a.vdim; d += 256) {
         float v = 0.0f;
-        for (int s = 0; s < a.nsplit; s++) { const float ms = a.part_ml[(base + s) * 2]; if (ms != -INFINITY) v = __builtin_fmaf(a.part_acc[(base + s) * a.vdim + d], expf(ms - M), v); }
-        sv_st(o + d, v / L);
+#pragma unroll 8
+        for (int s = 0; s < a.nsplit; s++) { const float w = wsp[s], p = a.part_acc[(base + s) * a.vdim + d]; v = __builtin_fmaf(w != 0.0f ? p : 0.0f, w, v); }      // a split without keys counts as zeros
+        sv_st(o + d, v * inv);
     }
 }
 
@@ -949,8 +959,8 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
     if (a.T <= 0) return;
     if (f32 ? sv_attn_mfma_launch<float>(a, st) : sv_attn_mfma_launch<uint16_t>(a, st)) {
         if (a.nsplit > 1) {
-            if (f32) hipLaunchKernelGGL(sv_attn_merge_kernel<float>, dim3(a.T, a.heads), dim3(64), 0, st, a);
-            else hipLaunchKernelGGL(sv_attn_merge_kernel<uint16_t>, dim3(a.T, a.heads), dim3(64), 0, st, a);
+            if (f32) hipLaunchKernelGGL(sv_attn_merge_kernel<float>, dim3(a.T, a.heads), dim3(256), (size_t)(a.nsplit + 1) * sizeof(float), st, a);
+            else hipLaunchKernelGGL(sv_attn_merge_kernel<uint16_t>, dim3(a.T, a.heads), dim3(256), (size_t)(a.nsplit + 1) * sizeof(float), st, a);
         }
         return;
     }
@@ -967,8 +977,8 @@ void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st) {
                           else { if (rm == 2) SV_ATT(T_, 2, 8); else SV_ATT(T_, 4, 8); } } while (0)
     if (f32) SV_ATT_T(float); else SV_ATT_T(uint16_t);
     if (a.nsplit > 1) {
-        if (f32) hipLaunchKernelGGL(sv_attn_merge_kernel<float>, dim3(a.T, a.heads), dim3(64), 0, st, a);
-        else hipLaunchKernelGGL(sv_attn_merge_kernel<uint16_t>, dim3(a.T, a.heads), dim3(64), 0, st, a);
+        if (f32) hipLaunchKernelGGL(sv_attn_merge_kernel<float>, dim3(a.T, a.heads), dim3(256), (size_t)(a.nsplit + 1) * sizeof(float), st, a);
+        else hipLaunchKernelGGL(sv_attn_merge_kernel<uint16_t>, dim3(a.T, a.heads), dim3(256), (size_t)(a.nsplit + 1) * sizeof(float), st, a);
     }
 #undef SV_ATT_T
 #undef SV_ATT_R
