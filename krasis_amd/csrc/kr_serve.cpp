@@ -570,7 +570,8 @@ int kr_serve_step(kr_serve* s, int n_entries, const int* slots, const int* count
     for (int li = 0; li < c.n_layers; li++) {
         const SvLayer& l = s->L[li]; const kr_serve_layer& d = l.d;
         const int visible = d.window > 0 ? std::min(max_pos + 1, d.window) : (d.chunk > 0 ? std::min(max_pos + 1, d.chunk) : max_pos + 1);
-        nsplit[li] = kr_sv_attention_splits(T, d.heads, l.att_heads_kv(), l.att_vdim(), visible);
+        const int ldk = l.latent() ? l.att_dim() : d.kv_heads * d.dim, ldv = l.latent() ? l.att_dim() : d.kv_heads * d.vdim;
+        nsplit[li] = kr_sv_attention_splits(T, d.heads, l.att_heads_kv(), l.att_dim(), l.att_vdim(), ldk, ldv, s->f32, visible);
         if (nsplit[li] > 1 && (s->part_ml.ensure(Ts * d.heads * nsplit[li] * 8) || s->part_acc.ensure(Ts * d.heads * nsplit[li] * l.att_vdim() * 4)))
             return kr_fail(KR_ERR_HIP, "attention split scratch");
     }

@@ -60,7 +60,7 @@ struct KrSvAttn {
     int tq;                          // set by the launcher of the matrix-instruction form: tokens per workgroup
 };
 // how many ways to split: fills the chip when the step has few tokens; max_visible = most keys any token of the step sees in this layer
-int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_visible);
+int kr_sv_attention_splits(int T, int heads, int kv_heads, int dim, int vdim, int ldk, int ldv, bool f32, int max_visible);
 void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st);      // rotation, unit norm, cache append
 void kr_sv_attention(const KrSvAttn& a, bool f32, hipStream_t st);   // windowed softmax with an optional sink over the paged cache
 

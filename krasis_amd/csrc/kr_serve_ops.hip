@@ -390,7 +390,7 @@ __global__ void __launch_bounds__(256) sv_attn_group_kernel(const KrSvAttn a) {
 // so a lane's accumulators all belong to ONE row and the online-softmax rescale is a per-lane scalar.  The reduction index of an MFMA is spread over the
 // four 16-lane groups; group q takes the CONTIGUOUS quarter q of a key row (dim / 4 elements, 16-byte loads) and the keys 4 q .. 4 q + 3 of a 16-key block.
 typedef float sv_f4 __attribute__((ext_vector_type(4)));
-template <typename T, int DQ, int DB>      // DQ = dim / 4 query elements per lane, DB = vdim / 16 value columns per lane
+template <typename T, int DQ, int DB, int NKB = 4>      // DQ = dim / 4 query elements per lane, DB = vdim / 16 value columns per lane, NKB = blocks of 16 keys a wave takes at a time
 __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int VEC = 16 / sizeof(T);
@@ -401,7 +401,11 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
     const int g = blockIdx.y, h_row = g * R + hb * 16 + (row % Rb), t0 = blockIdx.x * TQ, tq_row = row / Rb;
     float* ml = lds;                    // [4 waves][16 rows][2]
     float* mf = lds + 4 * 16 * 2;       // [16 rows][2]: the merged maximum and 1 / denominator (or the denominator itself in a split launch)
-    float* accs = mf + 16 * 2;          // [16 rows][vdim]
+    // [16 rows][AS]: a row is vdim + 65 floats long and the column block of lane group qd starts 16 floats late, so that the 64 lanes of a wave, which hold the
+    // same column of 16 rows x 4 groups, fall into distinct LDS banks (rows of exactly vdim floats put all of them into ONE bank)
+    float* accs = mf + 16 * 2;
+    constexpr int AS = DB * 16 + 65;
+    auto acc_at = [](int r, int c) { return r * AS + c + (c / (4 * DB)) * 16; };
     const T* kp = (const T*)a.kpool; const T* vp = (const T*)a.vpool;
     for (int base = 0; base < TQ && t0 + base < a.T;) {
         // the run of tokens [base, end) of this group that continue one request (same slot, consecutive positions)
@@ -424,19 +428,20 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
         sv_f4 acc[DB];
 #pragma unroll
         for (int d = 0; d < DB; d++) acc[d] = sv_f4{0.0f, 0.0f, 0.0f, 0.0f};
-        const int nch = (hi - lo) / 64 + 1, cps = (nch + a.nsplit - 1) / a.nsplit, c0 = sp * cps, c1 = min(nch, c0 + cps);
+        constexpr int KEYS = 16 * NKB;
+        const int nch = (hi - lo) / KEYS + 1, cps = (nch + a.nsplit - 1) / a.nsplit, c0 = sp * cps, c1 = min(nch, c0 + cps);
         for (int cb = c0 + wave; cb < c1; cb += 4) {
-            const int j0 = lo + 64 * cb;
-            // ---- S^T: four blocks of 16 keys
-            sv_f4 st[4];
-            int prow[4];
+            const int j0 = lo + KEYS * cb;
+            // ---- S^T: NKB blocks of 16 keys
+            sv_f4 st[NKB];
+            int prow[NKB];
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++) {
+            for (int kb = 0; kb < NKB; kb++) {
                 const int key = min(j0 + kb * 16 + row, hi);         // keys past the last one are fetched again and masked
                 prow[kb] = table[key / a.page_tokens] * a.page_tokens + (key % a.page_tokens);
             }
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++) {
+            for (int kb = 0; kb < NKB; kb++) {
                 const T* k = kp + (size_t)prow[kb] * a.ldk + (size_t)g * dim + qd * DQ;
                 // a key row's quarter in batches of at most PB 16-byte pieces: long rows (a latent cache row) must not hold all of it in registers at once
                 constexpr int NP = DQ / VEC, PB = NP <= 8 ? NP : 6;
@@ -466,7 +471,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             // ---- masks and the online softmax of this lane's row (its 16 keys here, the other 48 in the three lanes 16 apart)
             float cm = -INFINITY;
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++)
+            for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int key = j0 + kb * 16 + 4 * qd + i;
@@ -479,7 +484,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             const float alpha = mn == -INFINITY ? 1.0f : expf(m - mn);       // a row that has seen no key yet keeps its zero state
             float ps = 0.0f;
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++)
+            for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) { const float pj = st[kb][i] == -INFINITY ? 0.0f : expf(st[kb][i] - mn); st[kb][i] = pj; ps += pj; }
             ps += __shfl_xor(ps, 16); ps += __shfl_xor(ps, 32);
@@ -490,7 +495,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             // wide values (DB > 16) go through in column batches of DC, so that one batch of four keys' values is in registers at a time
             constexpr int DC = DB <= 16 ? DB : 8;
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++) {
+            for (int kb = 0; kb < NKB; kb++) {
                 int prk[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) prk[i] = __shfl(prow[kb], 4 * qd + i);
@@ -547,7 +552,7 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const int col = (4 * qd + i) * DB + d;
-                        accs[row * vdim + col] = (w == 0 ? 0.0f : accs[row * vdim + col]) + acc[d][i] * f;
+                        accs[acc_at(row, col)] = (w == 0 ? 0.0f : accs[acc_at(row, col)]) + acc[d][i] * f;
                     }
             }
             __syncthreads();
@@ -556,10 +561,11 @@ __global__ void __launch_bounds__(256) sv_attn_mfma_kernel(const KrSvAttn a) {
             const int r = i / vdim, tq = r / Rb;
             if (tq < base || tq >= end) continue;
             const int h = g * R + hb * 16 + (r % Rb);
-            if (last) sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), accs[i] * mf[r * 2 + 1]);
+            const float av = accs[acc_at(r, i - r * vdim)];
+            if (last) sv_st((T*)a.out + ((size_t)(t0 + tq) * a.heads + h) * vdim + (i - r * vdim), av * mf[r * 2 + 1]);
             else {
                 const size_t slot = ((size_t)(t0 + tq) * a.heads + h) * a.nsplit + sp;
-                a.part_acc[slot * vdim + (i - r * vdim)] = accs[i];
+                a.part_acc[slot * vdim + (i - r * vdim)] = av;
                 if (i == r * vdim) { a.part_ml[slot * 2] = mf[r * 2]; a.part_ml[slot * 2 + 1] = mf[r * 2 + 1]; }
             }
         }
@@ -907,14 +913,35 @@ void kr_sv_qk_prep(const KrSvAttn& a, bool f32, hipStream_t st) {
     else hipLaunchKernelGGL(sv_qk_prep_kernel<uint16_t>, grid, dim3(64), lds, st, a);
 }
 
-int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_visible) {
+// the register tilings of the matrix-instruction attention: (dim / 4, vdim / 16)
+static bool sv_mfma_tiling(int dq, int db) {
+    static const int tab[][2] = {{16, 4}, {32, 8}, {16, 8}, {32, 4}, {8, 2}, {8, 4}, {16, 2}, {64, 16}, {64, 8}, {32, 16}, {8, 16}, {8, 1}, {16, 1},
+                                 // latent cache rows: [latent | rotated part] as the key, the latent as the value (512 + 64, 256 + 64, 128 + 64 and the like)
+                                 {144, 32}, {80, 16}, {48, 8}};
+    for (const auto& t : tab) if (t[0] == dq && t[1] == db) return true;
+    return false;
+}
+static bool sv_mfma_fits(int heads, int kv_heads, int dim, int vdim, int ldk, int ldv, bool f32) {
+    const int VEC = f32 ? 4 : 8, R = heads / kv_heads;
+    if (!((R <= 16 && 16 % R == 0) || R % 16 == 0)) return false;
+    if (dim % (4 * VEC) != 0 || vdim % 16 != 0 || ldk % VEC != 0 || ldv % VEC != 0) return false;
+    return sv_mfma_tiling(dim / 4, vdim / 16);
+}
+// keys a wave takes at a time in a split launch: long rows on the matrix path go 16 at a time (a wave's loads of one 64-key block are ~40 dependent
+// batches at one wave per SIMD: a decode step is over sooner with four times the waves), everything else 64
+static int sv_split_key_block(int heads, int kv_heads, int dim, int vdim, int ldk, int ldv, bool f32) {
+    return (dim >= 192 && sv_mfma_fits(heads, kv_heads, dim, vdim, ldk, ldv, f32)) ? 16 : 64;
+}
+
+int kr_sv_attention_splits(int T, int heads, int kv_heads, int dim, int vdim, int ldk, int ldv, bool f32, int max_visible) {
     const int R = heads / kv_heads;
     const int vc = vdim <= 64 ? 1 : vdim <= 128 ? 2 : vdim <= 256 ? 4 : 8;
     const int rmax = vc <= 2 ? 16 : vc == 4 ? 8 : 4;
     int rm = 2;
     while (rm < R && rm < rmax) rm *= 2;
     const long blocks = (long)T * kv_heads * ((R + rm - 1) / rm);
-    const int nch = (max_visible + 63) / 64;
+    const int kblk = sv_split_key_block(heads, kv_heads, dim, vdim, ldk, ldv, f32);
+    const int nch = (max_visible + kblk - 1) / kblk;
     long ns = 1024 / (blocks > 0 ? blocks : 1);              // about four workgroups per compute unit
     if (ns > (nch + 3) / 4) ns = (nch + 3) / 4;              // a workgroup keeps at least one block of keys per wave
     return ns < 1 ? 1 : (int)ns;
@@ -923,16 +950,16 @@ int kr_sv_attention_splits(int T, int heads, int kv_heads, int vdim, int max_vis
 // the matrix-instruction form takes prompt-sized steps whose head sizes fit its register tiling
 template <typename T>
 static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
-    constexpr int VEC = 16 / sizeof(T);
+    if (!sv_mfma_fits(a.heads, a.kv_heads, a.dim, a.vdim, a.ldk, a.ldv, sizeof(T) == 4)) return false;
     const int R = a.heads / a.kv_heads;
-    if (!((R <= 16 && 16 % R == 0) || R % 16 == 0)) return false;
-    if (a.dim % (4 * VEC) != 0 || a.vdim % 16 != 0 || a.ldk % VEC != 0 || a.ldv % VEC != 0) return false;
     const int Rb = R < 16 ? R : 16;
     KrSvAttn b = a;
     b.tq = a.nsplit > 1 ? 1 : 16 / Rb;      // a split launch is a decode-shaped step: its tokens belong to different requests
     const dim3 grid((a.T + b.tq - 1) / b.tq, a.kv_heads, (R <= 16 ? 1 : R / 16) * a.nsplit);
-    const size_t lds = (size_t)(4 * 16 * 2 + 16 * 2 + 16 * a.vdim) * sizeof(float);
+    const size_t lds = (size_t)(4 * 16 * 2 + 16 * 2 + 16 * (a.vdim + 65)) * sizeof(float);
 #define SV_MF(DQ_, DB_) do { hipLaunchKernelGGL((sv_attn_mfma_kernel<T, DQ_, DB_>), grid, dim3(256), lds, st, b); return true; } while (0)
+#define SV_MF1(DQ_, DB_) do { if (a.nsplit > 1) hipLaunchKernelGGL((sv_attn_mfma_kernel<T, DQ_, DB_, 1>), grid, dim3(256), lds, st, b); \
+                              else hipLaunchKernelGGL((sv_attn_mfma_kernel<T, DQ_, DB_>), grid, dim3(256), lds, st, b); return true; } while (0)
     const int dq = a.dim / 4, db = a.vdim / 16;
     if (dq == 16 && db == 4) SV_MF(16, 4);
     if (dq == 32 && db == 8) SV_MF(32, 8);
@@ -947,11 +974,11 @@ static bool sv_attn_mfma_launch(const KrSvAttn& a, hipStream_t st) {
     if (dq == 8 && db == 16) SV_MF(8, 16);
     if (dq == 8 && db == 1) SV_MF(8, 1);
     if (dq == 16 && db == 1) SV_MF(16, 1);
-    // latent cache rows: [latent | rotated part] as the key, the latent as the value (512 + 64, 256 + 64, 128 + 64, 64 + 64 and the like)
-    if (dq == 144 && db == 32) SV_MF(144, 32);
-    if (dq == 80 && db == 16) SV_MF(80, 16);
-    if (dq == 48 && db == 8) SV_MF(48, 8);
+    if (dq == 144 && db == 32) SV_MF1(144, 32);     // split launches of the long rows: 16 keys per wave at a time (sv_split_key_block)
+    if (dq == 80 && db == 16) SV_MF1(80, 16);
+    if (dq == 48 && db == 8) SV_MF1(48, 8);
 #undef SV_MF
+#undef SV_MF1
     return false;
 }
 
