@@ -1,7 +1,8 @@
 """The batched serving store (kr_serve_*) with the Pamulix design against the plain float64 restatement in tests/oracle_pamulix.py.
 
 Small random models of several shapes; every comparison is between what the store's step function returns (logits, or the residual stream after each
-layer) and the oracle run on the whole sequence.  The f32 store is held to 2e-4 of the stream's scale, the bf16 store to 4e-2."""
+layer) and the oracle run on the whole sequence.  The f32 store is held to 2e-4 of the stream's scale; the bf16 store is judged row by row (typical
+row within 3 %), since a router's close call may fall the other way for single tokens."""
 import json
 import os
 import subprocess
